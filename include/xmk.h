@@ -1,0 +1,187 @@
+/*
+ * xmk.h — C ABI of the MI355X (gfx950) kernels behind the XLA custom calls
+ *         "__cublas$gemm", "__cublas$lt$matmul", "__cudnn$fmhaSoftmax",
+ *         "__cudnn$fmhaScaleBiasSoftmax" and the two weight-quantised targets
+ *         this library adds ("__xmk$int4_gemm", "__cublas$lt$matmul$f8").
+ *
+ * Plain pointers and sizes only.  Every `stream` argument is a hipStream_t
+ * passed as void* (NULL = the null stream).  Every entry point enqueues work
+ * on that stream and returns; none synchronises the device, none allocates
+ * device memory, none frees or retains a caller's buffer.
+ *
+ * Return value: 0 on success, otherwise an absl::StatusCode-compatible code
+ * (see xmk_status).  The message of the last failure on the calling thread is
+ * returned by xmk_last_error().
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   xla/service/gpu/sycl_custom_call.cc:154-226      FFI handlers (GEMM)
+ *   xla/service/gpu/sycl_onednn.cc:38-54             RunGemmCustomCall
+ *   xla/service/gpu/onednn_matmul_utils.h:35-73      epilogue enum + RunGemm
+ *   xla/service/gpu/matrix_descriptor.h:30-46        MatrixDescriptor
+ *   xla/service/gpu/xetla/gemm/gemm.h:57-108         XetlaGemmKernel builder
+ *   xla/service/gpu/xetla/sdp/sdp_forward.h:22-36    fmha_forward_kernel_*
+ *   xla/service/gpu/xetla_gpu_fused_mha_runner.h:36-41  RunXetlaGpuFMHA
+ */
+#ifndef XMK_H_
+#define XMK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes: the subset of absl::StatusCode the reference path returns
+ * (onednn_matmul_utils.cc:322,334,613; xetla_gpu_fused_mha_runner.cc:60,145,217). */
+typedef enum xmk_status {
+  XMK_OK = 0,
+  XMK_INVALID_ARGUMENT = 3,
+  XMK_UNIMPLEMENTED = 12,
+  XMK_INTERNAL = 13
+} xmk_status;
+
+/* Element types, numbered as xla::PrimitiveType (the values the reference's
+ * attribute dictionary carries in "{lhs,rhs,output}_layout_dtype",
+ * onednn_matmul_utils.cc:592-610). */
+typedef enum xmk_dtype {
+  XMK_S8 = 2,
+  XMK_S32 = 4,
+  XMK_F16 = 10,
+  XMK_F32 = 11,
+  XMK_BF16 = 16,
+  XMK_F8E4M3FN = 20
+} xmk_dtype;
+
+/* Epilogues, numbered as SYCLGemm::GemmBackendEpilogue
+ * (onednn_matmul_utils.h:35-45). */
+typedef enum xmk_epilogue {
+  XMK_EPI_DEFAULT = 0,
+  XMK_EPI_RELU = 1,
+  XMK_EPI_GELU = 2,
+  XMK_EPI_BIAS = 3,
+  XMK_EPI_BIAS_RELU = 4,
+  XMK_EPI_BIAS_GELU = 5,
+  XMK_EPI_GELU_AUX = 6,      /* rejected: XMK_UNIMPLEMENTED, as in the reference */
+  XMK_EPI_BIAS_GELU_AUX = 7  /* rejected: XMK_UNIMPLEMENTED, as in the reference */
+} xmk_epilogue;
+
+/* Mirrors xla::gpu::MatrixDescriptor (matrix_descriptor.h:30-46) with the
+ * device pointer flattened.  The buffer holds a row-major
+ * [num_rows, num_cols] matrix whose rows are leading_dim_stride elements
+ * apart; transpose != 0 means the operand of the product is the transpose of
+ * that stored matrix (what GetMatrixDesc, onednn_matmul_utils.cc:206-218,
+ * produces for a column-major layout). */
+typedef struct xmk_matrix {
+  void* data;
+  int32_t transpose;
+  int64_t num_rows;
+  int64_t num_cols;
+  int64_t batch_stride;       /* elements between consecutive batch members */
+  int64_t leading_dim_stride; /* elements between consecutive stored rows */
+} xmk_matrix;
+
+/* One GEMM custom call, after the attribute dictionary has been decoded
+ * (RunGemm, onednn_matmul_utils.cc:533-621):
+ *     out = act(alpha * lhs·rhs + beta * c + bias)
+ * computed with fp32 accumulation and one rounding to dtype_out.
+ * c may alias out.data.  bias is a length-n vector of dtype_in or NULL.
+ * Dtype triples accepted (onednn_matmul_utils.cc:605-610):
+ *   (BF16,BF16,BF16) (F16,F16,F16) (BF16,BF16,F32) (F16,F16,F32) (F32,F32,F32). */
+typedef struct xmk_gemm_desc {
+  xmk_matrix lhs;
+  xmk_matrix rhs;
+  xmk_matrix out;
+  const void* c;     /* matrix addend, laid out like out; NULL iff beta == 0 */
+  const void* bias;  /* vector addend; required iff the epilogue adds a bias */
+  int32_t dtype_in;  /* xmk_dtype of lhs, rhs, bias */
+  int32_t dtype_out; /* xmk_dtype of out and c */
+  int64_t batch_size;
+  float alpha;
+  float beta;
+  int32_t epilogue;  /* xmk_epilogue */
+} xmk_gemm_desc;
+
+/* Library version and the message of the calling thread's last failure. */
+const char* xmk_version(void);
+const char* xmk_last_error(void);
+
+/* Replaces RunGemm (onednn_matmul_utils.h:58-73) and everything under it
+ * (DoGemm :493-511, RunXetlaGemm :245-324, XetlaGemmKernel::run gemm.cc:315-325,
+ * hgemm_* hgemm_impl.h:101-459).  The MFMA kernel takes the cases the
+ * reference's XeTLA path takes (gemm.h:82-102: batch 1, alpha 1, A row-major,
+ * 16-bit in == out type); every other accepted combination runs a generic
+ * tiled kernel, where the reference falls back to oneDNN. */
+int xmk_gemm(const xmk_gemm_desc* desc, void* stream);
+
+/* Name of the tile policy xmk_gemm would pick for (m, n, k): the counterpart
+ * of selectXetlaGemmConfig (xetla/gemm/gemm.cc:286-308).  Returns a static
+ * string. */
+const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int32_t rhs_transpose,
+                                 int32_t dtype_in, int32_t dtype_out);
+
+/* Fused multi-head-attention forward.  Replaces fmha_forward_kernel_fp16 /
+ * _bf16 (xetla/sdp/sdp_forward.h:22-36; same argument meaning and order apart
+ * from the queue becoming a trailing stream, the dtype becoming an argument,
+ * dropout being dropped because the reference rejects it
+ * (xetla_gpu_fused_mha_runner.cc:59-61), and `causal` being a run-time flag
+ * where the reference hard-codes false, sdp_forward.cc:41).
+ *   query [B,N,F,H], key [B,N,T,H], value [B,N,T,H], out [B,N,F,H], all
+ *   H-contiguous and packed; bias [B,N,F,T] of the same dtype or NULL
+ *   (added after scaling, fmha_forward.h:266-281); lse fp32 [B*N,F] or NULL
+ *   (written as m + log l, fmha_forward.h:433-450).
+ *   causal != 0 masks key x > query y, top-left aligned (fmha_utils.h:45-96).
+ * dtype is XMK_F16 or XMK_BF16; 1 <= H <= 256. */
+int xmk_fmha_fwd(const void* query, const void* key, const void* value, const void* bias,
+                 void* out, float* lse, int32_t dtype, uint32_t num_batches,
+                 uint32_t num_heads, uint32_t head_size, uint32_t num_queries,
+                 uint32_t num_keys, float head_scale, int32_t causal, void* stream);
+
+/* Bytes of device workspace xmk_fmha_decode needs for the given shape. */
+size_t xmk_fmha_decode_workspace_bytes(uint32_t num_batches, uint32_t num_heads,
+                                       uint32_t head_size, uint32_t num_keys);
+
+/* Attention for one query row per (batch, head) (num_queries == 1), with the
+ * keys split over work-groups and merged by a second pass.  Same tensors as
+ * xmk_fmha_fwd with F = 1; key/value may sit in a cache whose rows per head
+ * are kv_head_stride elements apart (>= T*H).  The reference has no such
+ * kernel: it would run fmha_forward with a 64-row tile (fmha_forward.h:633-640). */
+int xmk_fmha_decode(const void* query, const void* key, const void* value, void* out,
+                    int32_t dtype, uint32_t num_batches, uint32_t num_heads,
+                    uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
+                    float head_scale, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Int4 weight-only GEMM (not in the reference snapshot; the contract is this
+ * header's):
+ *   qweight int32 [K/8, N]: nibble j (bits 4j..4j+3) of qweight[r, n] is the
+ *     unsigned 4-bit weight of input channel k = 8r + j, output channel n;
+ *   scales, zeros fp16 [K/group, N];
+ *   W[k, n] = fp16( (float(q) - float(zeros[k/group, n])) * float(scales[k/group, n]) )
+ *     with a separate fp32 subtract and fp32 multiply, rounded to nearest even;
+ *   out[m, n] = fp16( sum_k float(act[m, k]) * float(W[k, n]) + float(bias[n]) ),
+ *     fp32 accumulation; bias fp16 [N] or NULL.
+ * act fp16 [M, K] packed, out fp16 [M, N] packed.  K % group == 0,
+ * group % 8 == 0, N % 8 == 0. */
+int xmk_int4_gemm(const void* act, const void* qweight, const void* scales, const void* zeros,
+                  const void* bias, void* out, int64_t m, int64_t k, int64_t n,
+                  int64_t group, void* stream);
+
+/* The dequantised weight matrix itself, fp16 [K, N]: the bit-exact check
+ * surface for the formula above. */
+int xmk_int4_dequant(const void* qweight, const void* scales, const void* zeros, void* w_out,
+                     int64_t k, int64_t n, int64_t group, void* stream);
+
+/* FP8 GEMM (not in the reference snapshot; follows XLA's
+ * "__cublas$lt$matmul$f8" convention):
+ *   out[m, n] = bf16( a_scale * b_scale * sum_k float(a[m,k]) * float(b) ), fp32 accumulate.
+ * a e4m3fn [M, K] row-major; b e4m3fn, [K, N] row-major when
+ * rhs_transpose == 0 or [N, K] row-major when rhs_transpose != 0;
+ * a_scale, b_scale device pointers to one fp32 each; out bf16 [M, N]. */
+int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                 void* out, int64_t m, int64_t n, int64_t k, int32_t rhs_transpose,
+                 void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XMK_H_ */
