@@ -156,12 +156,14 @@ int xmk_fmha_decode(const void* query, const void* key, const void* value, void*
  *   qweight int32 [K/8, N]: nibble j (bits 4j..4j+3) of qweight[r, n] is the
  *     unsigned 4-bit weight of input channel k = 8r + j, output channel n;
  *   scales, zeros fp16 [K/group, N];
- *   W[k, n] = fp16( (float(q) - float(zeros[k/group, n])) * float(scales[k/group, n]) )
- *     with a separate fp32 subtract and fp32 multiply, rounded to nearest even;
- *   out[m, n] = fp16( sum_k float(act[m, k]) * float(W[k, n]) + float(bias[n]) ),
- *     fp32 accumulation; bias fp16 [N] or NULL.
- * act fp16 [M, K] packed, out fp16 [M, N] packed.  K % group == 0,
- * group % 8 == 0, N % 8 == 0. */
+ *   w[k, n] = (float(q) - float(zeros[k/group, n])) * float(scales[k/group, n])
+ *     with a separate fp32 subtract and fp32 multiply;
+ *   W[k, n] = fp16(w[k, n]), rounded to nearest even, is what xmk_int4_dequant writes;
+ *   out[m, n] = fp16( sum_k float(act[m, k]) * w[k, n] + float(bias[n]) ),
+ *     fp32 accumulation, no intermediate rounding of w to fp16; bias fp16 [N] or NULL.
+ * act fp16 [M, K] packed, out fp16 [M, N] packed.  K % group == 0, N % 8 == 0;
+ * group is 32, 64, 128 or 256 for xmk_int4_gemm and any multiple of 8 for
+ * xmk_int4_dequant. */
 int xmk_int4_gemm(const void* act, const void* qweight, const void* scales, const void* zeros,
                   const void* bias, void* out, int64_t m, int64_t k, int64_t n,
                   int64_t group, void* stream);

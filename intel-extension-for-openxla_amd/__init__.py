@@ -1,0 +1,193 @@
+"""MI355X (gfx950) kernels behind the XLA custom calls of the reference PJRT plugin.
+
+The product is ``libxmk.so`` (``include/xmk.h``): hand-written HIP kernels behind a
+C ABI.  This module is the thin ctypes binding the tests and the benchmark use;
+torch only supplies device memory and the stream.  There is no CPU fallback: if
+the library is missing or a call fails, the wrappers raise.
+
+Function names follow the reference's host entry points:
+``run_gemm`` <-> RunGemm (xla/service/gpu/onednn_matmul_utils.h:58-73),
+``fmha_forward`` <-> fmha_forward_kernel_{fp16,bf16} (xla/service/gpu/xetla/sdp/sdp_forward.h:22-36).
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libxmk.so")
+
+# xla::PrimitiveType numbering
+S8, S32, F16, F32, BF16, F8E4M3FN = 2, 4, 10, 11, 16, 20
+# SYCLGemm::GemmBackendEpilogue numbering (onednn_matmul_utils.h:35-45)
+(EPI_DEFAULT, EPI_RELU, EPI_GELU, EPI_BIAS, EPI_BIAS_RELU, EPI_BIAS_GELU, EPI_GELU_AUX,
+ EPI_BIAS_GELU_AUX) = range(8)
+
+OK, INVALID_ARGUMENT, UNIMPLEMENTED, INTERNAL = 0, 3, 12, 13
+
+_TORCH_DTYPE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32,
+                torch.float8_e4m3fn: F8E4M3FN, torch.int8: S8, torch.int32: S32}
+
+
+class XmkError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"xmk status {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+class Matrix(ctypes.Structure):
+    """xmk_matrix (mirrors xla::gpu::MatrixDescriptor, matrix_descriptor.h:30-46)."""
+    _fields_ = [("data", ctypes.c_void_p), ("transpose", ctypes.c_int32),
+                ("num_rows", ctypes.c_int64), ("num_cols", ctypes.c_int64),
+                ("batch_stride", ctypes.c_int64), ("leading_dim_stride", ctypes.c_int64)]
+
+
+class GemmDesc(ctypes.Structure):
+    """xmk_gemm_desc."""
+    _fields_ = [("lhs", Matrix), ("rhs", Matrix), ("out", Matrix), ("c", ctypes.c_void_p),
+                ("bias", ctypes.c_void_p), ("dtype_in", ctypes.c_int32),
+                ("dtype_out", ctypes.c_int32), ("batch_size", ctypes.c_int64),
+                ("alpha", ctypes.c_float), ("beta", ctypes.c_float), ("epilogue", ctypes.c_int32)]
+
+
+_lib = None
+
+
+def lib():
+    """Loads libxmk.so; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is missing: run `python {_HERE}/build.py` "
+                               "(there is no CPU fallback)")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, restype in (("xmk_version", ctypes.c_char_p),
+                              ("xmk_last_error", ctypes.c_char_p),
+                              ("xmk_gemm_policy_name", ctypes.c_char_p),
+                              ("xmk_fmha_decode_workspace_bytes", ctypes.c_size_t)):
+            if hasattr(L, name):
+                getattr(L, name).restype = restype
+        _lib = L
+    return _lib
+
+
+def _check(code):
+    if code != 0:
+        raise XmkError(code, lib().xmk_last_error().decode())
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(stream=None):
+    s = torch.cuda.current_stream() if stream is None else stream
+    return ctypes.c_void_p(s.cuda_stream)
+
+
+def dtype_code(t):
+    return _TORCH_DTYPE[t.dtype]
+
+
+def version():
+    return lib().xmk_version().decode()
+
+
+# ----------------------------------------------------------------------- GEMM
+def matrix(t, transpose=False, batch_stride=None):
+    """Describes a 2-D (or batched 3-D) row-major tensor as an xmk_matrix."""
+    rows, cols = t.shape[-2], t.shape[-1]
+    ld = t.stride(-2)
+    bs = (t.stride(0) if t.dim() == 3 else 0) if batch_stride is None else batch_stride
+    return Matrix(t.data_ptr(), int(bool(transpose)), rows, cols, bs, ld)
+
+
+def run_gemm_desc(desc, stream=None):
+    _check(lib().xmk_gemm(ctypes.byref(desc), _stream(stream)))
+
+
+def run_gemm(lhs, rhs, out, *, lhs_transpose=False, rhs_transpose=False, out_transpose=False,
+             c=None, bias=None, alpha=1.0, beta=0.0, epilogue=EPI_DEFAULT, stream=None):
+    """out = act(alpha * op(lhs) op(rhs) + beta * c + bias).  Tensors are the *stored*
+    row-major matrices; ``*_transpose`` marks the operand as the transpose of what is
+    stored (a column-major XLA layout)."""
+    batch = lhs.shape[0] if lhs.dim() == 3 else 1
+    d = GemmDesc(matrix(lhs, lhs_transpose), matrix(rhs, rhs_transpose),
+                 matrix(out, out_transpose), None if c is None else c.data_ptr(),
+                 None if bias is None else bias.data_ptr(), dtype_code(lhs), dtype_code(out),
+                 batch, alpha, beta, epilogue)
+    run_gemm_desc(d, stream)
+    return out
+
+
+def gemm_policy_name(m, n, k, rhs_transpose=False, dtype_in=BF16, dtype_out=BF16):
+    return lib().xmk_gemm_policy_name(ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
+                                      ctypes.c_int32(int(rhs_transpose)), ctypes.c_int32(dtype_in),
+                                      ctypes.c_int32(dtype_out)).decode()
+
+
+# ------------------------------------------------------------------ attention
+def fmha_forward(query, key, value, out, *, bias=None, lse=None, head_scale=None, causal=False,
+                 stream=None):
+    """query [B,N,F,H], key/value [B,N,T,H], out [B,N,F,H]; bias [B,N,F,T]; lse fp32 [B*N,F]."""
+    B, N, F, H = query.shape
+    T = key.shape[2]
+    scale = (H ** -0.5) if head_scale is None else head_scale
+    _check(lib().xmk_fmha_fwd(_ptr(query), _ptr(key), _ptr(value), _ptr(bias), _ptr(out),
+                              _ptr(lse), ctypes.c_int32(dtype_code(query)), ctypes.c_uint32(B),
+                              ctypes.c_uint32(N), ctypes.c_uint32(H), ctypes.c_uint32(F),
+                              ctypes.c_uint32(T), ctypes.c_float(scale),
+                              ctypes.c_int32(int(causal)), _stream(stream)))
+    return out
+
+
+def fmha_decode_workspace_bytes(B, N, H, T):
+    return lib().xmk_fmha_decode_workspace_bytes(ctypes.c_uint32(B), ctypes.c_uint32(N),
+                                                 ctypes.c_uint32(H), ctypes.c_uint32(T))
+
+
+def fmha_decode(query, key, value, out, workspace, *, num_keys=None, kv_head_stride=None,
+                head_scale=None, stream=None):
+    """query/out [B,N,1,H] (or [B,N,H]); key/value [B,N,Tcap,H] caches of which the first
+    ``num_keys`` rows are attended."""
+    B, N = query.shape[0], query.shape[1]
+    H = query.shape[-1]
+    T = key.shape[2] if num_keys is None else num_keys
+    stride = key.stride(1) if kv_head_stride is None else kv_head_stride
+    scale = (H ** -0.5) if head_scale is None else head_scale
+    _check(lib().xmk_fmha_decode(_ptr(query), _ptr(key), _ptr(value), _ptr(out),
+                                 ctypes.c_int32(dtype_code(query)), ctypes.c_uint32(B),
+                                 ctypes.c_uint32(N), ctypes.c_uint32(H), ctypes.c_uint32(T),
+                                 ctypes.c_int64(stride), ctypes.c_float(scale), _ptr(workspace),
+                                 ctypes.c_size_t(workspace.numel() * workspace.element_size()),
+                                 _stream(stream)))
+    return out
+
+
+# ----------------------------------------------------------------------- int4
+def int4_gemm(act, qweight, scales, zeros, out, *, group=128, bias=None, stream=None):
+    m, k = act.shape
+    n = qweight.shape[1]
+    _check(lib().xmk_int4_gemm(_ptr(act), _ptr(qweight), _ptr(scales), _ptr(zeros), _ptr(bias),
+                               _ptr(out), ctypes.c_int64(m), ctypes.c_int64(k), ctypes.c_int64(n),
+                               ctypes.c_int64(group), _stream(stream)))
+    return out
+
+
+def int4_dequant(qweight, scales, zeros, w_out, *, group=128, stream=None):
+    k, n = qweight.shape[0] * 8, qweight.shape[1]
+    _check(lib().xmk_int4_dequant(_ptr(qweight), _ptr(scales), _ptr(zeros), _ptr(w_out),
+                                  ctypes.c_int64(k), ctypes.c_int64(n), ctypes.c_int64(group),
+                                  _stream(stream)))
+    return w_out
+
+
+# ------------------------------------------------------------------------ fp8
+def fp8_gemm(a, b, a_scale, b_scale, out, *, rhs_transpose=False, stream=None):
+    m, k = a.shape
+    n = b.shape[0] if rhs_transpose else b.shape[1]
+    _check(lib().xmk_fp8_gemm(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(out),
+                              ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
+                              ctypes.c_int32(int(rhs_transpose)), _stream(stream)))
+    return out

@@ -178,7 +178,9 @@ def int4_dequant(qweight, scales, zeros, group):
     return out
 
 
-def int4_gemm(act, qweight, scales, zeros, group, bias=None):
+def int4_gemm(act, qweight, scales, zeros, group, bias=None, round_weights=False):
+    """round_weights=False: the GEMM contract (fp32 dequantised weights); True: weights rounded
+    to fp16 first, i.e. act @ int4_dequant(...)."""
     act = np.ascontiguousarray(act, dtype=np.uint16)
     qweight = np.ascontiguousarray(qweight, dtype=np.uint32)
     m, k = act.shape
@@ -187,7 +189,7 @@ def int4_gemm(act, qweight, scales, zeros, group, bias=None):
     out_f32 = np.empty((m, n), dtype=np.float32)
     lib().xo_int4_gemm(_p(act), _p(qweight), _p(scales), _p(zeros), _p(bias), _p(out),
                        _p(out_f32), ctypes.c_int64(m), ctypes.c_int64(k), ctypes.c_int64(n),
-                       ctypes.c_int64(group))
+                       ctypes.c_int64(group), ctypes.c_int(int(round_weights)))
     return out, out_f32
 
 

@@ -328,10 +328,13 @@ void xo_int4_dequant(const uint32_t* qweight, const uint16_t* scales, const uint
                                       scales[g * n + j], zeros[g * n + j]);
   }
 }
-/* out[m,n] = f16(sum_k f32(act[m,k]) * f32(W[k,n]) + f32(bias[n])), double accumulation. */
+/* out[m,n] = f16(sum_k f32(act[m,k]) * w[k,n] + f32(bias[n])), double accumulation, where
+ * w[k,n] is the dequantised weight: the fp32 value (f32(q) - f32(z)) * f32(s) when
+ * round_weights == 0 (the GEMM's contract: no intermediate rounding to fp16), or that value
+ * rounded to fp16 (the output of xo_int4_dequant) when round_weights != 0. */
 void xo_int4_gemm(const uint16_t* act, const uint32_t* qweight, const uint16_t* scales,
                   const uint16_t* zeros, const uint16_t* bias, uint16_t* out, float* out_f32,
-                  int64_t m, int64_t k, int64_t n, int64_t group) {
+                  int64_t m, int64_t k, int64_t n, int64_t group, int round_weights) {
   float* af = (float*)malloc(sizeof(float) * (size_t)(m * k));
   for (int64_t i = 0; i < m * k; ++i) af[i] = xo_f16_to_f32(act[i]);
 #pragma omp parallel for schedule(static)
@@ -339,8 +342,16 @@ void xo_int4_gemm(const uint16_t* act, const uint32_t* qweight, const uint16_t* 
     double* acc = (double*)calloc((size_t)m, sizeof(double));
     for (int64_t kk = 0; kk < k; ++kk) {
       int64_t g = kk / group;
-      float w = xo_f16_to_f32(dequant_one(qweight[(kk / 8) * n + j], (int)(kk % 8),
-                                          scales[g * n + j], zeros[g * n + j]));
+      uint32_t word = qweight[(kk / 8) * n + j];
+      float w;
+      if (round_weights) {
+        w = xo_f16_to_f32(dequant_one(word, (int)(kk % 8), scales[g * n + j], zeros[g * n + j]));
+      } else {
+        float q = (float)((word >> (4 * (kk % 8))) & 0xfu);
+        volatile float d = q - xo_f16_to_f32(zeros[g * n + j]);
+        volatile float wv = d * xo_f16_to_f32(scales[g * n + j]);
+        w = wv;
+      }
       for (int64_t i = 0; i < m; ++i) acc[i] += (double)af[i * k + kk] * (double)w;
     }
     for (int64_t i = 0; i < m; ++i) {

@@ -1,0 +1,197 @@
+"""GPU parity: bf16/fp16 GEMM with fused epilogue through the C ABI (xmk_gemm), against the oracle.
+
+Tolerance (BASELINE north star): max relative error <= 1e-2 for bf16/fp16 outputs against an
+fp32 recompute from the same rounded inputs; both normalisations of oracle.rel_err are held to it.
+"""
+import numpy as np
+import pytest
+import torch
+
+from util import to_bits, to_dev
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _kind(dt, oracle):
+    return "bf16" if dt == oracle.BF16 else "f16"
+
+
+def _check(oracle, got_f32, ref_f32, tol=TOL):
+    g, e = oracle.rel_err(got_f32, ref_f32)
+    assert g <= tol and e <= tol, (g, e)
+    return g, e
+
+
+def test_config1_bf16_bias(xmk, oracle):
+    """BASELINE config 1: C[512,4096] = A[512,4096] B[4096,4096] + bias, N(0,1)/sqrt(K) inputs."""
+    m, k, n = 512, 4096, 4096
+    sc = k ** -0.5
+    a = oracle.from_f32(oracle.normal((m, k), 1, sc), oracle.BF16)
+    b = oracle.from_f32(oracle.normal((k, n), 2, sc), oracle.BF16)
+    bias = oracle.from_f32(oracle.normal((n,), 3, sc), oracle.BF16)
+    _, ref = oracle.gemm_packed(a, b, oracle.BF16, oracle.BF16, bias=bias, epilogue=oracle.EPI_BIAS)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    xmk.run_gemm(to_dev(a, "bf16"), to_dev(b, "bf16"), out, bias=to_dev(bias, "bf16"),
+                 epilogue=xmk.EPI_BIAS)
+    torch.cuda.synchronize()
+    g, e = _check(oracle, out.float().cpu().numpy(), ref)
+    print(f"config1: global {g:.2e} elementwise {e:.2e}")
+
+
+@pytest.mark.parametrize("dt_name", ["BF16", "F16"])
+@pytest.mark.parametrize("lhs_t,rhs_t,out_t", [(0, 0, 0), (0, 1, 0), (1, 0, 0), (1, 1, 0), (0, 0, 1), (1, 0, 1)])
+@pytest.mark.parametrize("m,n,k", [(96, 136, 200), (300, 264, 72), (256, 256, 64)])
+def test_layouts(xmk, oracle, dt_name, lhs_t, rhs_t, out_t, m, n, k):
+    """Row/column-major operands and output (MakeBlasGemmCompatible), ragged tiles, K tails."""
+    dt = getattr(oracle, dt_name)
+    kind = _kind(dt, oracle)
+    a = oracle.from_f32(oracle.normal((k, m) if lhs_t else (m, k), 10, 0.3), dt)
+    b = oracle.from_f32(oracle.normal((n, k) if rhs_t else (k, n), 11, 0.3), dt)
+    ref_bits, ref = oracle.gemm(a, b, dt, dt, lhs_t=lhs_t, rhs_t=rhs_t, out_t=out_t)
+    tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+    out = torch.full((n, m) if out_t else (m, n), float("nan"), dtype=tdt, device="cuda")
+    xmk.run_gemm(to_dev(a, kind), to_dev(b, kind), out, lhs_transpose=lhs_t, rhs_transpose=rhs_t,
+                 out_transpose=out_t)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    _check(oracle, got.T if out_t else got, ref[0])
+
+
+@pytest.mark.parametrize("epi", ["DEFAULT", "RELU", "GELU", "BIAS", "BIAS_RELU", "BIAS_GELU"])
+@pytest.mark.parametrize("beta", [0.0, 1.0, 0.5])
+def test_epilogues(xmk, oracle, epi, beta):
+    """out = act(A.B + beta*C + bias) with C aliasing the output (sycl_custom_call.cc:191-195)."""
+    dt = oracle.BF16
+    m, n, k = 200, 328, 256
+    a = oracle.from_f32(oracle.normal((m, k), 20, 0.2), dt)
+    b = oracle.from_f32(oracle.normal((k, n), 21, 0.2), dt)
+    bias = oracle.from_f32(oracle.normal((n,), 22), dt)
+    c = oracle.from_f32(oracle.normal((m, n), 23), dt)
+    code = getattr(oracle, "EPI_" + epi)
+    _, ref = oracle.gemm(a, b, dt, dt, bias=bias, c=c if beta else None, beta=beta, epilogue=code)
+    out = to_dev(c, "bf16") if beta else torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    xmk.run_gemm(to_dev(a, "bf16"), to_dev(b, "bf16"), out, c=out if beta else None,
+                 bias=to_dev(bias, "bf16") if "BIAS" in epi else None, beta=beta,
+                 epilogue=getattr(xmk, "EPI_" + epi))
+    torch.cuda.synchronize()
+    _check(oracle, out.float().cpu().numpy(), ref[0])
+
+
+def test_identity_is_bit_exact(xmk, oracle):
+    dt = oracle.BF16
+    m, k = 320, 256
+    a = oracle.from_f32(oracle.normal((m, k), 30), dt)
+    eye = to_dev(oracle.from_f32(np.eye(k, dtype=np.float32), dt), "bf16")
+    out = torch.empty((m, k), dtype=torch.bfloat16, device="cuda")
+    xmk.run_gemm(to_dev(a, "bf16"), eye, out)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_bits(out), a)
+
+
+@pytest.mark.parametrize("dt_name", ["BF16", "F16"])
+@pytest.mark.parametrize("shape", [(1, 256, 128, 8), (1, 1024, 64, 128)])
+def test_reference_gemm_ut_shapes(xmk, oracle, dt_name, shape):
+    """Shapes of the reference's gemm_ut (test/jax_ut.patch:505-518): B column-major, GELU epilogue."""
+    _, m, k, n = shape
+    dt = getattr(oracle, dt_name)
+    kind = _kind(dt, oracle)
+    a = oracle.from_f32(oracle.normal((m, k), 40, 0.1), dt)
+    bt = oracle.from_f32(oracle.normal((n, k), 41, 0.1), dt)
+    _, ref = oracle.gemm(a, bt, dt, dt, rhs_t=True, epilogue=oracle.EPI_GELU)
+    out = torch.empty((m, n), dtype=torch.bfloat16 if kind == "bf16" else torch.float16, device="cuda")
+    xmk.run_gemm(to_dev(a, kind), to_dev(bt, kind), out, rhs_transpose=True, epilogue=xmk.EPI_GELU)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    _check(oracle, got, ref[0])
+    if dt == oracle.F16:  # the reference's own bound for fp16 (test/jax_ut.patch:614)
+        assert np.abs(got - ref[0]).max() < 1e-3
+
+
+def test_batched_f32_out_and_strides(xmk, oracle):
+    dt = oracle.F16
+    bsz, m, n, k = 3, 72, 88, 128
+    a = oracle.from_f32(oracle.normal((bsz, m, k), 50, 0.2), dt)
+    b = oracle.from_f32(oracle.normal((bsz, k, n), 51, 0.2), dt)
+    _, ref = oracle.gemm(a, b, dt, oracle.F32)
+    out = torch.empty((bsz, m, n), dtype=torch.float32, device="cuda")
+    xmk.run_gemm(to_dev(a, "f16"), to_dev(b, "f16"), out)
+    torch.cuda.synchronize()
+    _check(oracle, out.cpu().numpy(), ref, tol=1e-4)  # fp32 output: accumulation-order noise only
+    # padded leading dimensions: views into wider buffers
+    ap = torch.zeros((m, k + 24), dtype=torch.float16, device="cuda")
+    bp = torch.zeros((k, n + 40), dtype=torch.float16, device="cuda")
+    op = torch.full((m, n + 8), 7.0, dtype=torch.float16, device="cuda")
+    ap[:, :k] = to_dev(a[0], "f16")
+    bp[:, :n] = to_dev(b[0], "f16")
+    xmk.run_gemm(ap[:, :k], bp[:, :n], op[:, :n])
+    torch.cuda.synchronize()
+    _check(oracle, op[:, :n].float().cpu().numpy(), ref[0])
+    assert (op[:, n:] == 7.0).all()  # nothing written outside the logical matrix
+
+
+def test_generic_path(xmk, oracle):
+    """Shapes and types the MFMA kernel does not take: K % 8 != 0, fp32, s8 -> s32."""
+    dt = oracle.BF16
+    m, n, k = 37, 50, 45
+    a = oracle.from_f32(oracle.normal((m, k), 60, 0.3), dt)
+    b = oracle.from_f32(oracle.normal((k, n), 61, 0.3), dt)
+    bias = oracle.from_f32(oracle.normal((n,), 62), dt)
+    _, ref = oracle.gemm(a, b, dt, dt, bias=bias, epilogue=oracle.EPI_BIAS_GELU)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    assert xmk.gemm_policy_name(m, n, k, dtype_in=xmk.F32, dtype_out=xmk.F32) == "generic_64x64"
+    xmk.run_gemm(to_dev(a, "bf16"), to_dev(b, "bf16"), out, bias=to_dev(bias, "bf16"),
+                 epilogue=xmk.EPI_BIAS_GELU)
+    torch.cuda.synchronize()
+    _check(oracle, out.float().cpu().numpy(), ref[0])
+    af, bf = oracle.normal((m, k), 63), oracle.normal((n, k), 64)
+    outf = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    xmk.run_gemm(to_dev(af, "f32"), to_dev(bf, "f32"), outf, rhs_transpose=True)
+    torch.cuda.synchronize()
+    assert np.allclose(outf.cpu().numpy(), af.astype(np.float64) @ bf.T.astype(np.float64), rtol=1e-4, atol=1e-4)
+    ai = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
+    bi = torch.randint(-128, 128, (k, n), dtype=torch.int8, device="cuda")
+    oi = torch.empty((m, n), dtype=torch.int32, device="cuda")
+    xmk.run_gemm(ai, bi, oi)
+    torch.cuda.synchronize()
+    assert torch.equal(oi.cpu(), ai.cpu().int() @ bi.cpu().int())  # integer path: bit exact
+
+
+@pytest.mark.parametrize("rhs_t", [False, True])
+def test_full_size_8192_sampled_rows(xmk, oracle, rhs_t):
+    """The 8192^3 shape of the north-star target: every 512th output row against the oracle."""
+    n = 8192
+    sc = n ** -0.5
+    a = oracle.from_f32(oracle.normal((n, n), 70, sc), oracle.BF16)
+    b = oracle.from_f32(oracle.normal((n, n), 71, sc), oracle.BF16)
+    out = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+    xmk.run_gemm(to_dev(a, "bf16"), to_dev(b, "bf16"), out, rhs_transpose=rhs_t)
+    torch.cuda.synchronize()
+    rows = np.arange(5, n, 512)
+    _, ref = oracle.gemm_packed(a[rows], b, oracle.BF16, oracle.BF16, rhs_t=rhs_t)
+    _check(oracle, out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), ref)
+    # checksum of checksums: sum of every output row equals A @ rowsum(B) (linearity), fp64 on host
+    bs = oracle.to_f32(b, oracle.BF16).astype(np.float64)
+    colsum = bs.sum(axis=0 if rhs_t else 1)
+    expect = oracle.to_f32(a, oracle.BF16).astype(np.float64) @ colsum
+    got = out.double().sum(dim=1).cpu().numpy()
+    assert np.abs(got - expect).max() <= 2e-2 * np.abs(expect).max() + 0.5
+
+
+def test_errors(xmk):
+    a = torch.zeros((16, 32), dtype=torch.bfloat16, device="cuda")
+    b = torch.zeros((32, 16), dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros((16, 16), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.run_gemm(a, b, out, epilogue=xmk.EPI_GELU_AUX)
+    assert e.value.code == xmk.UNIMPLEMENTED and "Unsupported Activation mode" in e.value.message
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.run_gemm(a, b, out, epilogue=xmk.EPI_BIAS)  # bias missing
+    assert e.value.code == xmk.INVALID_ARGUMENT
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.run_gemm(a, a, out)  # reduction sizes differ
+    assert e.value.code == xmk.INVALID_ARGUMENT
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.run_gemm(a, b, out.float().half())  # bf16 x bf16 -> f16 is not an accepted triple
+    assert e.value.code == xmk.INTERNAL

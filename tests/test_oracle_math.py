@@ -138,9 +138,19 @@ def test_int4_gemm(oracle):
     bias = oracle.from_f32(oracle.normal((n,), 34), oracle.F16)
     w = _np_dequant(qw, s, z, 128).astype(np.float64)
     ref = act.view(np.float16).astype(np.float64) @ w + bias.view(np.float16).astype(np.float64)
-    out, f32 = oracle.int4_gemm(act, qw, s, z, 128, bias=bias)
+    out, f32 = oracle.int4_gemm(act, qw, s, z, 128, bias=bias, round_weights=True)
     assert np.allclose(f32, ref, rtol=1e-6, atol=1e-6)
     assert np.array_equal(out, f32.astype(np.float16).view(np.uint16))
+    # the GEMM contract proper: fp32 dequantised weights, no fp16 rounding in between
+    qf = ((np.repeat(qw, 8, axis=0) >> (4 * (np.arange(k) % 8).astype(np.uint32)[:, None])) & 0xF)
+    zf = np.repeat(z.view(np.float16).astype(np.float32), 128, axis=0)
+    sf = np.repeat(s.view(np.float16).astype(np.float32), 128, axis=0)
+    w32 = ((qf.astype(np.float32) - zf).astype(np.float32) * sf).astype(np.float32)
+    ref32 = (act.view(np.float16).astype(np.float64) @ w32.astype(np.float64)
+             + bias.view(np.float16).astype(np.float64))
+    _, f32u = oracle.int4_gemm(act, qw, s, z, 128, bias=bias)
+    assert np.allclose(f32u, ref32, rtol=1e-6, atol=1e-6)
+    assert oracle.rel_err(f32u, f32)[0] < 2e-3  # the two definitions differ by fp16 weight rounding only
 
 
 # ------------------------------------------------------------------------ fp8
