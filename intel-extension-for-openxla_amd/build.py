@@ -1,6 +1,6 @@
 """Builds libxmk.so (the C-ABI kernel library) for gfx950 with hipcc, in-tree.
 
-Usage: python build.py [-j N]
+Usage: python build.py [-j N] [--force]   (without --force: incremental)
 Each translation unit under csrc/ is compiled to an object file and the objects
 are linked into one shared library next to this file.
 """
@@ -26,8 +26,19 @@ def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith((".hip", ".cc")))
 
 
-def _compile(src):
+def _deps_mtime():
+    hdrs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    hdrs += [os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE)]
+    return max(os.path.getmtime(h) for h in hdrs)
+
+
+def _compile(args):
+    src, force = args
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
+    spath = os.path.join(CSRC, src)
+    if (not force and os.path.exists(obj)
+            and os.path.getmtime(obj) > max(os.path.getmtime(spath), _deps_mtime())):
+        return src, obj, 0, ""
     cmd = [HIPCC] + FLAGS + (["-x", "hip"] if src.endswith(".cc") else []) + \
           ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -36,12 +47,13 @@ def _compile(src):
     return src, obj, r.returncode, out
 
 
-def build(jobs=None, verbose=False):
+def build(jobs=None, verbose=False, force=True):
+    """force=False recompiles only sources newer than their object file."""
     os.makedirs(OBJ, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     objs = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        for src, obj, rc, out in pool.map(_compile, sources()):
+        for src, obj, rc, out in pool.map(_compile, [(s, force) for s in sources()]):
             if out and (verbose or rc != 0):
                 print(f"--- {src}\n{out}", file=sys.stderr)
             if rc != 0:
@@ -54,4 +66,4 @@ def build(jobs=None, verbose=False):
 
 if __name__ == "__main__":
     j = int(sys.argv[sys.argv.index("-j") + 1]) if "-j" in sys.argv else None
-    print(build(j, verbose=True))
+    print(build(j, verbose=True, force="--force" in sys.argv))

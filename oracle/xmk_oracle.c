@@ -403,10 +403,12 @@ int xo_fp8_gemm(const uint8_t* a, const uint8_t* b, float a_scale, float b_scale
 void xo_fmha_fwd(int dtype, const void* q, const void* k, const void* v, const void* bias,
                  void* out, float* out_f32, float* lse, int64_t num_units, int64_t first_unit,
                  int64_t H, int64_t F, int64_t T, int64_t kv_unit_stride, float scale,
-                 int causal) {
+                 int causal, int64_t f_stride) {
+  /* f_stride > 1: only query rows 0, f_stride, 2 f_stride, ... are computed (sampling). */
 #pragma omp parallel for schedule(dynamic, 1) collapse(2)
   for (int64_t u = first_unit; u < first_unit + num_units; ++u) {
     for (int64_t f = 0; f < F; ++f) {
+      if (f % f_stride != 0) continue;
       double* s = (double*)malloc(sizeof(double) * (size_t)T);
       double* o = (double*)calloc((size_t)H, sizeof(double));
       float* qf = (float*)malloc(sizeof(float) * (size_t)H);

@@ -1,0 +1,119 @@
+"""GPU parity: fused multi-head-attention forward through the C ABI (xmk_fmha_fwd) against the
+oracle's closed form.  Tolerance: max relative error <= 1e-2 (bf16/fp16), plus the reference
+test's own absolute bound (test/jax_ut.patch:997: atol 3e-2 bf16, 1e-2 fp16)."""
+import numpy as np
+import pytest
+import torch
+
+from util import to_bits, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _dt(oracle, name):
+    return (oracle.BF16, "bf16", torch.bfloat16) if name == "bf16" else (oracle.F16, "f16", torch.float16)
+
+
+def _run(xmk, oracle, name, B, N, F, T, H, *, causal=False, use_bias=False, lse=False, seed=0,
+         units=None, f_stride=1, scale=None):
+    dt, kind, tdt = _dt(oracle, name)
+    q = oracle.from_f32(oracle.normal((B, N, F, H), seed + 1), dt)
+    k = oracle.from_f32(oracle.normal((B, N, T, H), seed + 2), dt)
+    v = oracle.from_f32(oracle.normal((B, N, T, H), seed + 3), dt)
+    bias = oracle.from_f32(oracle.normal((B, N, F, T), seed + 4), dt) if use_bias else None
+    scale = H ** -0.5 if scale is None else scale
+    out = torch.full((B, N, F, H), float("nan"), dtype=tdt, device="cuda")
+    lse_t = torch.full((B * N, F), float("nan"), dtype=torch.float32, device="cuda") if lse else None
+    xmk.fmha_forward(to_dev(q, kind), to_dev(k, kind), to_dev(v, kind), out,
+                     bias=None if bias is None else to_dev(bias, kind), lse=lse_t,
+                     head_scale=scale, causal=causal)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy().reshape(B * N, F, H)
+    assert np.isfinite(got).all()
+    units = list(range(B * N)) if units is None else units
+    for u in units:
+        _, ref, ref_lse = oracle.fmha_fwd(q, k, v, dt, scale, bias=bias, causal=causal, want_lse=True,
+                                          first_unit=u, num_units=1, f_stride=f_stride)
+        ref = ref.reshape(B * N, F, H)[u, ::f_stride]
+        g, e = oracle.rel_err(got[u, ::f_stride], ref)
+        assert g <= 1e-2 and e <= 1e-2, (u, g, e)
+        assert np.abs(got[u, ::f_stride] - ref).max() <= (3e-2 if name == "bf16" else 1e-2)
+        if lse:
+            gl = lse_t.cpu().numpy()[u, ::f_stride]
+            assert np.allclose(gl, ref_lse[u, ::f_stride], rtol=1e-3, atol=1e-3)
+    return out
+
+
+def test_config2_causal_bf16(xmk, oracle):
+    """BASELINE config 2: bf16 [8,32,2048,128], causal, scale 1/sqrt(128); three units, every 8th row."""
+    _run(xmk, oracle, "bf16", 8, 32, 2048, 2048, 128, causal=True, units=[0, 101, 255], f_stride=8)
+
+
+def test_config2_full_size_properties(xmk, oracle):
+    """Size-independent properties at the full shape: V = 1 => O = 1; causal row 0 == V[0]."""
+    B, N, S, H = 8, 32, 2048, 128
+    q = torch.randn((B, N, S, H), device="cuda").bfloat16()
+    k = torch.randn((B, N, S, H), device="cuda").bfloat16()
+    ones = torch.ones((B, N, S, H), device="cuda").bfloat16()
+    out = torch.empty_like(q)
+    xmk.fmha_forward(q, k, ones, out, causal=True)
+    torch.cuda.synchronize()
+    assert (out.float() - 1.0).abs().max().item() <= 1e-2
+    v = torch.randn((B, N, S, H), device="cuda").bfloat16()
+    xmk.fmha_forward(q, k, v, out, causal=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out[:, :, 0, :], v[:, :, 0, :])
+
+
+SD_SHAPES = [  # (b, F, T, heads, head_dim) of the reference's mha_rewrite_test (test/jax_ut.patch:914-935)
+    (2, 9216, 9216, 5, 64), (2, 9216, 77, 5, 64), (2, 2304, 2304, 10, 64), (2, 2304, 77, 10, 64),
+    (2, 576, 576, 20, 64), (2, 576, 77, 20, 64), (2, 144, 144, 20, 64), (2, 144, 77, 20, 64),
+    (2, 4096, 4096, 8, 40), (2, 4096, 77, 8, 40), (2, 4096, 4096, 10, 64), (2, 4096, 77, 10, 64),
+    (2, 1024, 1024, 8, 80), (2, 1024, 77, 8, 80), (2, 1024, 1024, 20, 64), (2, 1024, 77, 20, 64),
+    (2, 256, 256, 8, 160), (2, 256, 77, 8, 160), (2, 64, 64, 8, 160), (2, 64, 77, 8, 160),
+]
+
+
+@pytest.mark.parametrize("name", ["bf16", "fp16"])
+@pytest.mark.parametrize("shape", SD_SHAPES)
+def test_reference_mha_shapes(xmk, oracle, name, shape):
+    """The reference's 20 shapes x 2 dtypes, no mask, no bias, scale head_dim**-0.5.  Large shapes
+    are checked on two units and a stride of query rows so the oracle finishes in seconds."""
+    b, F, T, n, h = shape
+    work = F * T
+    f_stride = 1 if work <= (1 << 20) else (16 if work <= (1 << 24) else 128)
+    units = [0, b * n - 1] if work > (1 << 18) else None
+    _run(xmk, oracle, name, b, n, F, T, h, units=units, f_stride=f_stride, seed=F + T)
+
+
+@pytest.mark.parametrize("name", ["bf16", "fp16"])
+@pytest.mark.parametrize("causal,use_bias", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("F,T,H", [(130, 200, 128), (64, 333, 64), (257, 129, 256), (1, 77, 80), (200, 64, 8)])
+def test_masks_bias_lse(xmk, oracle, name, causal, use_bias, F, T, H):
+    """Causal (top-left aligned, fmha_utils.h:45-96), additive bias [B,N,F,T], ragged F/T (padding
+    mask, fmha_forward.h:313-318), LSE output (fmha_forward.h:433-450)."""
+    _run(xmk, oracle, name, 2, 3, F, T, H, causal=causal, use_bias=use_bias, lse=True, seed=F * 7 + T)
+
+
+def test_key_permutation_invariance(xmk):
+    B, N, F, T, H = 1, 4, 256, 320, 128
+    q = torch.randn((B, N, F, H), device="cuda").bfloat16()
+    k = torch.randn((B, N, T, H), device="cuda").bfloat16()
+    v = torch.randn((B, N, T, H), device="cuda").bfloat16()
+    perm = torch.randperm(T, device="cuda")
+    o1, o2 = torch.empty_like(q), torch.empty_like(q)
+    xmk.fmha_forward(q, k, v, o1)
+    xmk.fmha_forward(q, k[:, :, perm].contiguous(), v[:, :, perm].contiguous(), o2)
+    torch.cuda.synchronize()
+    assert (o1.float() - o2.float()).abs().max().item() <= 2e-2
+
+
+def test_errors(xmk):
+    q = torch.zeros((1, 1, 8, 12), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.fmha_forward(q, q, q, q.clone())
+    assert e.value.code == xmk.UNIMPLEMENTED
+    q = torch.zeros((1, 1, 8, 16), dtype=torch.float32, device="cuda")
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.fmha_forward(q, q, q, q.clone())
+    assert e.value.code == xmk.INTERNAL and "Invalid MHA datatype" in e.value.message
