@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Roofline benchmark of the custom-call kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also] [--no-cpu]
+
+One JSON line on stdout.  A "step" is one launch of the workload's kernel on synthetic inputs that
+are already resident in HBM.  The headline workload is BASELINE config 2 (fused causal MHA forward,
+bf16 [8,32,2048,128]); the other configs are timed the same way and reported under "also".
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0}  # dense MFMA TFLOP/s, MI355X
+HBM_PEAK = 8000.0                                        # GB/s
+
+
+def _events(torch, fn, steps, warmup, graph=False):
+    """Average duration (ms) of fn over `steps` launches, HIP events on torch's current stream
+    (the stream every xmk call below is launched on).  graph=True replays the launches from one
+    captured HIP graph, so that kernels of a few microseconds are not timed at the rate the host
+    can enqueue them from Python."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(steps):
+                fn()
+        launches = fn
+        fn, steps_in = (lambda: g.replay()), steps
+        fn()  # one untimed replay
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        wall0 = time.perf_counter()
+        start.record()
+        fn()
+        stop.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - wall0) * 1e3 / steps_in
+        return start.elapsed_time(stop) / steps_in, wall
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - wall0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall
+
+
+# ---------------------------------------------------------------- workloads
+def wl_fmha(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
+    q, k, v = (torch.randn((B, N, S, H), device="cuda").bfloat16() for _ in range(3))
+    out = torch.empty_like(q)
+    flops = 4.0 * B * N * S * S * H * (0.5 if causal else 1.0)
+    nbytes = 4.0 * B * N * S * H * 2
+    name = f"fmha_fwd_{'causal_' if causal else ''}bf16_b{B}_h{N}_s{S}_d{H}"
+    return dict(name=name, fn=lambda: xmk.fmha_forward(q, k, v, out, causal=causal), flops=flops,
+                bytes=nbytes, bound="mfma", dtype="bf16", kernel="fmha_fwd_kernel",
+                note="causal FLOPs counted as 2*B*N*S^2*D (half of the dense 4*B*N*S^2*D)")
+
+
+def wl_gemm(torch, xmk, m, n, k, bias=False, rhs_t=False):
+    a = (torch.randn((m, k), device="cuda") * k ** -0.5).bfloat16()
+    b = (torch.randn((n, k) if rhs_t else (k, n), device="cuda") * k ** -0.5).bfloat16()
+    bv = (torch.randn((n,), device="cuda") * k ** -0.5).bfloat16() if bias else None
+    out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    epi = xmk.EPI_BIAS if bias else xmk.EPI_DEFAULT
+    return dict(name=f"gemm_bf16_{m}x{n}x{k}{'_bias' if bias else ''}{'_rhsT' if rhs_t else ''}",
+                fn=lambda: xmk.run_gemm(a, b, out, rhs_transpose=rhs_t, bias=bv, epilogue=epi),
+                flops=2.0 * m * n * k, bytes=2.0 * (m * k + k * n + m * n) + (2 * n if bias else 0),
+                bound="mfma", dtype="bf16", kernel="gemm_mfma_kernel")
+
+
+def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
+    # Rotate through `copies` weight sets (12 x 35.7 MB > the 256 MB last-level cache) so that
+    # every launch streams its weights from HBM.
+    qws = [torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 8, n), dtype=torch.int32, device="cuda")
+           for _ in range(copies)]
+    sc = [(torch.rand((k // group, n), device="cuda") * 0.019 + 0.001).half() for _ in range(copies)]
+    zp = [(torch.rand((k // group, n), device="cuda") * 15).half() for _ in range(copies)]
+    act = torch.randn((m, k), device="cuda").half()
+    out = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    state = [0]
+
+    def fn():
+        i = state[0] % copies
+        state[0] += 1
+        xmk.int4_gemm(act, qws[i], sc[i], zp[i], out, group=group)
+    nbytes = k * n / 2 + 2 * (k // group) * n * 2 + 2 * m * k + 2 * m * n
+    return dict(name=f"int4_gemm_m{m}_k{k}_n{n}_g{group}", fn=fn, flops=2.0 * m * k * n, bytes=nbytes,
+                bound="hbm", dtype="f16", kernel="int4_gemm_kernel", graph=True)
+
+
+WORKLOADS = {
+    "fmha_causal": lambda t, x: wl_fmha(t, x, True),
+    "fmha": lambda t, x: wl_fmha(t, x, False),
+    "gemm_8192": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192),
+    "gemm_8192_rhsT": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192, rhs_t=True),
+    "gemm_c1": lambda t, x: wl_gemm(t, x, 512, 4096, 4096, bias=True),
+    "int4_m1": lambda t, x: wl_int4(t, x, 1),
+    "int4_m8": lambda t, x: wl_int4(t, x, 8),
+    "int4_m32": lambda t, x: wl_int4(t, x, 32),
+}
+ALSO = ["gemm_8192", "gemm_c1", "int4_m1", "int4_m8", "int4_m32"]
+
+
+def measure(torch, xmk, key, steps, warmup):
+    w = WORKLOADS[key](torch, xmk)
+    ms, wall_ms = _events(torch, w["fn"], steps, warmup, graph=w.get("graph", False))
+    if w["bound"] == "mfma":
+        achieved, peak, unit = w["flops"] / ms / 1e9, PEAK["bf16"], "TFLOP/s"
+    else:
+        achieved, peak, unit = w["bytes"] / ms / 1e6, HBM_PEAK, "GB/s"
+    roof = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": None, "kernel": w["kernel"],
+            "kernel_ms": round(ms, 5), "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]}
+    return w, ms, wall_ms, roof
+
+
+def cpu_baseline_fmha(units=256, B=8, N=32, S=2048, H=128):
+    """The oracle (a CPU port of the path) on `units` of the workload's B*N (batch, head) units."""
+    import numpy as np
+    import oracle
+    rng_shape = (1, units, S, H)
+    q, k, v = (oracle.from_f32(oracle.normal(rng_shape, 5 + i), oracle.BF16) for i in range(3))
+    t0 = time.perf_counter()
+    oracle.fmha_fwd(q, k, v, oracle.BF16, H ** -0.5, causal=True)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * units * S * S * H
+    return {"value": round(flops / dt / 1e12, 6), "unit": "TFLOP/s", "cores": oracle.num_threads(),
+            "kind": "port", "seconds": round(dt, 2),
+            "sample": f"{units} of {B * N} (batch, head) units of the same causal bf16 "
+                      f"S={S} D={H} workload, oracle/xmk_oracle.c xo_fmha_fwd (OpenMP, double accumulation)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="fmha_causal", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-also", action="store_true", help="time only the headline workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    xmk = importlib.import_module("intel-extension-for-openxla_amd")
+    xmk.lib()  # fails loudly if libxmk.so is missing: there is no fallback path
+    torch.cuda.set_device(0)
+
+    w, ms, wall_ms, roof = measure(torch, xmk, args.workload, args.steps, args.warmup)
+    line = {
+        "metric": "TFLOP/s & %MFMA peak (GEMM/MHA); int4 GEMV HBM GB/s & %peak; 1 GPU",
+        "value": roof["achieved"], "unit": roof["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": w["name"], "note": w.get("note", "")},
+        "roofline": roof,
+    }
+    if not args.no_also:
+        also = {}
+        for key in ALSO:
+            if key == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            w2, ms2, _, roof2 = measure(torch, xmk, key, max(10, args.steps // 2), max(3, args.warmup // 2))
+            also[w2["name"]] = roof2
+        line["also"] = also
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_fmha()
+    try:
+        props = torch.cuda.get_device_properties(0)
+        line["device"] = {"name": props.name, "cus": props.multi_processor_count,
+                          "clock_mhz": getattr(props, "clock_rate", 0) // 1000}
+    except Exception:  # device query is informational only
+        pass
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -250,6 +250,10 @@ def fmha_fwd_online(q, k, v, dtype, scale, *, bias=None, causal=False, kBc=128):
     return out_f32
 
 
+def num_threads():
+    return int(lib().xo_num_threads())
+
+
 # ------------------------------------------------------------- error metrics
 def rel_err(x, ref):
     """Two readings of "max relative error" against the fp32 recompute ``ref``:

@@ -499,3 +499,11 @@ void xo_fmha_fwd_online(int dtype, const void* q, const void* k, const void* v, 
     }
   }
 }
+
+/* Threads the OpenMP loops above will use (reported as cpu_baseline.cores). */
+#ifdef _OPENMP
+#include <omp.h>
+int xo_num_threads(void) { return omp_get_max_threads(); }
+#else
+int xo_num_threads(void) { return 1; }
+#endif
