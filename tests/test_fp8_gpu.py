@@ -1,0 +1,55 @@
+"""GPU parity: FP8 (e4m3fn) GEMM through the C ABI (xmk_fp8_gemm) against the oracle.
+Tolerance: max relative error <= 5e-2 for fp8 outputs against an fp32 recompute of the same
+quantised inputs (the kernel accumulates exact products in fp32, so it lands far inside)."""
+import numpy as np
+import pytest
+import torch
+
+from util import to_bits, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _quant(oracle, shape, seed):
+    q, s = oracle.fp8_quantize(oracle.normal(shape, seed))
+    return q, s
+
+
+@pytest.mark.parametrize("m,n,k,rhs_t", [
+    (256, 256, 128, True), (512, 384, 1024, True), (300, 260, 208, True), (64, 8, 16, True),
+    (130, 72, 80, False), (256, 256, 256, False),
+])
+def test_fp8_gemm_shapes(xmk, oracle, m, n, k, rhs_t):
+    a, sa = _quant(oracle, (m, k), 1)
+    b, sb = _quant(oracle, (n, k) if rhs_t else (k, n), 2)
+    ref_bits, ref = oracle.fp8_gemm(a, b, sa, sb, rhs_t=rhs_t)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    xmk.fp8_gemm(to_dev(a, "f8"), to_dev(b, "f8"), torch.tensor([sa], device="cuda"),
+                 torch.tensor([sb], device="cuda"), out, rhs_transpose=rhs_t)
+    torch.cuda.synchronize()
+    g, e = oracle.rel_err(out.float().cpu().numpy(), ref)
+    assert g <= 5e-2 and e <= 5e-2, (g, e)
+    # exact fp8 products accumulated in fp32: what is left is the bf16 rounding of the output
+    assert g <= 5e-3 and e <= 5e-3, (g, e)
+
+
+def test_config4_fp8_8192_sampled_rows(xmk, oracle):
+    """BASELINE config 4: A, B [8192,8192] e4m3fn from N(0,1) with amax/448 scales, bf16 output."""
+    n = 8192
+    a, sa = _quant(oracle, (n, n), 11)
+    b, sb = _quant(oracle, (n, n), 12)  # stored [N, K]
+    out = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
+    xmk.fp8_gemm(to_dev(a, "f8"), to_dev(b, "f8"), torch.tensor([sa], device="cuda"),
+                 torch.tensor([sb], device="cuda"), out, rhs_transpose=True)
+    torch.cuda.synchronize()
+    rows = np.arange(3, n, 512)
+    _, ref = oracle.fp8_gemm(a[rows], b, sa, sb, rhs_t=True)
+    g, e = oracle.rel_err(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), ref)
+    print(f"config4 fp8: global {g:.2e} elementwise {e:.2e}")
+    assert g <= 5e-2 and e <= 5e-2
+    # identity-like property over the whole output: row sums equal A @ rowsum(B^T) (linearity)
+    table = oracle.to_f32(np.arange(256, dtype=np.uint8), oracle.F8E4M3FN).astype(np.float64)
+    colsum = table[b].sum(axis=0)
+    expect = (table[a] @ colsum) * float(sa) * float(sb)
+    got = out.double().sum(dim=1).cpu().numpy()
+    assert np.abs(got - expect).max() <= 2e-2 * np.abs(expect).max() + 1.0
