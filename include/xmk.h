@@ -183,6 +183,51 @@ int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, const float
                  void* out, int64_t m, int64_t n, int64_t k, int32_t rhs_transpose,
                  void* stream);
 
+/* ------------------------------------------------------------------------
+ * GPT-J-shaped decode step on int4 weights: one new token per sequence through
+ * n_layer blocks, reading the KV cache of the earlier positions.  The model the
+ * reference runs for this workload is FlaxGPTJForCausalLM under jax.jit
+ * (example/gptj/jax_gptj.py:57-68,94-97), with dense weights; the block structure
+ * restated here is GPT-J's: h = ln_1(x); x' = x + out_proj(attn(rotary(q), rotary(k), v))
+ * + fc_out(gelu_new(fc_in(h))); q/k/v/out_proj without bias, fc_in/fc_out/lm_head with
+ * bias; rotary on the first rotary_dim dims of each head, interleaved pairs, base 10000;
+ * scores scaled by 1/sqrt(head_dim); final ln_f then lm_head. */
+typedef struct xmk_int4_linear {
+  const void* qweight; /* int32 [k/8, n] */
+  const void* scales;  /* fp16 [k/group, n] */
+  const void* zeros;   /* fp16 [k/group, n] */
+  const void* bias;    /* fp16 [n] or NULL */
+  int64_t k, n;
+} xmk_int4_linear;
+
+typedef struct xmk_gptj_layer {
+  const void* ln_gamma; /* fp16 [d_model] */
+  const void* ln_beta;  /* fp16 [d_model] */
+  xmk_int4_linear qkv;      /* d_model -> 3 d_model, output columns [q | k | v], no bias */
+  xmk_int4_linear out_proj; /* d_model -> d_model, no bias */
+  xmk_int4_linear fc_in;    /* d_model -> d_ff, bias */
+  xmk_int4_linear fc_out;   /* d_ff -> d_model, bias */
+  void* k_cache; /* fp16 [batch, n_head, cache_capacity, head_dim]; row `position` is written */
+  void* v_cache; /* same */
+} xmk_gptj_layer;
+
+typedef struct xmk_gptj_config {
+  int32_t n_layer, n_head, head_dim, rotary_dim, d_model, d_ff, vocab, group;
+  int32_t batch, cache_capacity;
+  float ln_eps;
+} xmk_gptj_config;
+
+size_t xmk_gptj_decode_workspace_bytes(const xmk_gptj_config* cfg);
+
+/* hidden_in fp16 [batch, d_model] (the new token's embedding); position = index of the new
+ * token (the caches hold positions 0..position-1); logits fp16 [batch, vocab].
+ * Enqueues every kernel of the step on `stream` in order; a caller may capture the call in a
+ * HIP graph. */
+int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_layer* layers,
+                         const void* lnf_gamma, const void* lnf_beta,
+                         const xmk_int4_linear* lm_head, const void* hidden_in, int32_t position,
+                         void* logits, void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -191,3 +191,61 @@ def fp8_gemm(a, b, a_scale, b_scale, out, *, rhs_transpose=False, stream=None):
                               ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
                               ctypes.c_int32(int(rhs_transpose)), _stream(stream)))
     return out
+
+
+# ------------------------------------------------------------ GPT-J decode step
+class Int4Linear(ctypes.Structure):
+    """xmk_int4_linear."""
+    _fields_ = [("qweight", ctypes.c_void_p), ("scales", ctypes.c_void_p), ("zeros", ctypes.c_void_p),
+                ("bias", ctypes.c_void_p), ("k", ctypes.c_int64), ("n", ctypes.c_int64)]
+
+
+class GptjLayer(ctypes.Structure):
+    """xmk_gptj_layer."""
+    _fields_ = [("ln_gamma", ctypes.c_void_p), ("ln_beta", ctypes.c_void_p), ("qkv", Int4Linear),
+                ("out_proj", Int4Linear), ("fc_in", Int4Linear), ("fc_out", Int4Linear),
+                ("k_cache", ctypes.c_void_p), ("v_cache", ctypes.c_void_p)]
+
+
+class GptjConfig(ctypes.Structure):
+    """xmk_gptj_config."""
+    _fields_ = [(n, ctypes.c_int32) for n in ("n_layer", "n_head", "head_dim", "rotary_dim", "d_model",
+                                              "d_ff", "vocab", "group", "batch", "cache_capacity")] + \
+               [("ln_eps", ctypes.c_float)]
+
+
+def int4_linear(qweight, scales, zeros, bias=None):
+    return Int4Linear(qweight.data_ptr(), scales.data_ptr(), zeros.data_ptr(),
+                      None if bias is None else bias.data_ptr(), qweight.shape[0] * 8, qweight.shape[1])
+
+
+class GptjDecoder:
+    """Holds the descriptor arrays of a GPT-J-shaped int4 model and runs decode steps.
+
+    ``layers``: list of dicts with torch tensors ln_gamma, ln_beta, k_cache, v_cache and, for each
+    of qkv / out_proj / fc_in / fc_out, a tuple (qweight, scales, zeros, bias-or-None).
+    """
+
+    def __init__(self, cfg, layers, lnf_gamma, lnf_beta, lm_head):
+        self.cfg = cfg
+        self._keep = (layers, lnf_gamma, lnf_beta, lm_head)  # keep the tensors alive
+        arr = (GptjLayer * len(layers))()
+        for i, L in enumerate(layers):
+            arr[i] = GptjLayer(L["ln_gamma"].data_ptr(), L["ln_beta"].data_ptr(), int4_linear(*L["qkv"]),
+                               int4_linear(*L["out_proj"]), int4_linear(*L["fc_in"]),
+                               int4_linear(*L["fc_out"]), L["k_cache"].data_ptr(), L["v_cache"].data_ptr())
+        self.layers = arr
+        self.lnf = (lnf_gamma, lnf_beta)
+        self.lm_head = int4_linear(*lm_head)
+        lib().xmk_gptj_decode_workspace_bytes.restype = ctypes.c_size_t
+        nbytes = lib().xmk_gptj_decode_workspace_bytes(ctypes.byref(cfg))
+        if nbytes == 0:
+            raise XmkError(INVALID_ARGUMENT, lib().xmk_last_error().decode())
+        self.workspace = torch.empty((nbytes,), dtype=torch.uint8, device=lnf_gamma.device)
+
+    def step(self, hidden_in, position, logits, stream=None):
+        _check(lib().xmk_gptj_decode_step(ctypes.byref(self.cfg), self.layers, _ptr(self.lnf[0]),
+                                          _ptr(self.lnf[1]), ctypes.byref(self.lm_head), _ptr(hidden_in),
+                                          ctypes.c_int32(position), _ptr(logits), _ptr(self.workspace),
+                                          ctypes.c_size_t(self.workspace.numel()), _stream(stream)))
+        return logits

@@ -1,0 +1,241 @@
+// Attention for a single query row per (batch, head) unit (decode, seq_q = 1): HBM-bound
+// streaming of the K and V cache rows.
+//
+// The keys of a unit are split over `splits` work-groups so that a few dozen units still
+// fill 256 CUs (flash-decoding).  Pass 1 (fmha_decode_split_kernel): a work-group takes
+// one contiguous chunk of keys; lanes run along h (16 bytes each, a row is read as one
+// contiguous segment), scores are reduced across the lanes of a row with DPP/permute
+// shuffles, the chunk's softmax statistics are formed in LDS and the chunk's unnormalised
+// output  sum_t 2^(s_t - m) V[t,:]  is written to the workspace together with (m, l).
+// Pass 2 (fmha_decode_merge_kernel): one work-group per unit rescales and adds the
+// partial results and writes the output row.
+#include "common.h"
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int NT = 256;
+
+struct DecodeParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* ws;  // [units][splits][H + 2]: partial O (H floats), m, l
+  int N, H, T;
+  int64_t kv_head_stride;  // elements between consecutive heads' caches
+  int splits, chunk;
+  float scale2;
+};
+
+template <typename T>
+__device__ __forceinline__ void unpack8(u32x4 raw, float* f) {
+  union { u32x4 u; T e[8]; } x;
+  x.u = raw;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f[i] = (float)x.e[i];
+}
+
+// LPR: lanes per row (H <= 8 * LPR), a power of two <= 32.
+template <typename T, int LPR>
+__global__ __launch_bounds__(NT) void fmha_decode_split_kernel(DecodeParams p) {
+  constexpr int RPP = NT / LPR;  // rows per pass of the block
+  constexpr int MAXCH = 512;     // keys per chunk, upper bound
+  __shared__ float s_score[MAXCH];
+  __shared__ float s_red[NT / 64][8 * 32];  // per-wave partial outputs (up to 256 h)
+  __shared__ float s_stat[2];
+
+  const int tid = threadIdx.x;
+  const int unit = blockIdx.x / p.splits, split = blockIdx.x % p.splits;
+  const int t_begin = split * p.chunk;
+  const int t_end = min(p.T, t_begin + p.chunk);
+  const int nkeys = t_end - t_begin;  // may be <= 0 for trailing splits
+  const int H = p.H;
+  const int lr = tid % LPR, rr = tid / LPR;
+  const int h0 = lr * 8;
+  const bool h_ok = h0 < H;
+
+  const T* Q = reinterpret_cast<const T*>(p.q) + (int64_t)unit * H;
+  const int64_t kv_base = (int64_t)(unit / p.N) * p.N * p.kv_head_stride + (int64_t)(unit % p.N) * p.kv_head_stride;
+  const T* K = reinterpret_cast<const T*>(p.k) + kv_base;
+  const T* V = reinterpret_cast<const T*>(p.v) + kv_base;
+  float* wsu = p.ws + ((int64_t)unit * p.splits + split) * (H + 2);
+
+  float qf[8];
+  {
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (h_ok) raw = *reinterpret_cast<const u32x4*>(Q + h0);
+    unpack8<T>(raw, qf);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] *= p.scale2;
+  }
+
+  // ---- scores s_t = scale2 * q . k_t
+  for (int r0 = 0; r0 < nkeys; r0 += RPP * 4) {
+    u32x4 raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = r0 + j * RPP + rr;
+      raw[j] = u32x4{0u, 0u, 0u, 0u};
+      if (r < nkeys && h_ok) raw[j] = *reinterpret_cast<const u32x4*>(K + (int64_t)(t_begin + r) * H + h0);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float kf[8];
+      unpack8<T>(raw[j], kf);
+      float d = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) d = fmaf(qf[i], kf[i], d);
+#pragma unroll
+      for (int o = LPR / 2; o >= 1; o >>= 1) d += __shfl_xor(d, o);
+      const int r = r0 + j * RPP + rr;
+      if (lr == 0 && r < nkeys) s_score[r] = d;
+    }
+  }
+  __syncthreads();
+
+  // ---- chunk statistics: m = max s, p_t = 2^(s_t - m), l = sum p_t   (wave 0)
+  if (tid < 64) {
+    float m = -INFINITY;
+    for (int r = tid; r < nkeys; r += 64) m = fmaxf(m, s_score[r]);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    float l = 0.f;
+    for (int r = tid; r < nkeys; r += 64) {
+      const float e = __builtin_amdgcn_exp2f(s_score[r] - m);
+      s_score[r] = e;
+      l += e;
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) l += __shfl_xor(l, o);
+    if (tid == 0) { s_stat[0] = m; s_stat[1] = l; }
+  }
+  __syncthreads();
+
+  // ---- partial output: acc[h] = sum_t p_t V[t, h]
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int r0 = 0; r0 < nkeys; r0 += RPP * 4) {
+    u32x4 raw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = r0 + j * RPP + rr;
+      raw[j] = u32x4{0u, 0u, 0u, 0u};
+      if (r < nkeys && h_ok) raw[j] = *reinterpret_cast<const u32x4*>(V + (int64_t)(t_begin + r) * H + h0);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = r0 + j * RPP + rr;
+      const float pt = r < nkeys ? s_score[r] : 0.f;
+      float vf[8];
+      unpack8<T>(raw[j], vf);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(pt, vf[i], acc[i]);
+    }
+  }
+  // Rows of one wave that share h: lanes lr, lr + LPR, ... -> reduce inside the wave, then over waves.
+#pragma unroll
+  for (int o = 32; o >= LPR; o >>= 1)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], o);
+  const int wave = tid >> 6, lane = tid & 63;
+  if (lane < LPR) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s_red[wave][lane * 8 + i] = acc[i];
+  }
+  __syncthreads();
+  for (int h = tid; h < H; h += NT) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < NT / 64; ++w) s += s_red[w][h];
+    wsu[h] = s;
+  }
+  if (tid == 0) { wsu[H] = s_stat[0]; wsu[H + 1] = s_stat[1]; }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void fmha_decode_merge_kernel(DecodeParams p) {
+  const int unit = blockIdx.x, H = p.H;
+  const float* wsu = p.ws + (int64_t)unit * p.splits * (H + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < p.splits; ++s) m = fmaxf(m, wsu[(int64_t)s * (H + 2) + H]);
+  float l = 0.f;
+  for (int s = 0; s < p.splits; ++s) {
+    const float ms = wsu[(int64_t)s * (H + 2) + H];
+    if (ms > -INFINITY) l += wsu[(int64_t)s * (H + 2) + H + 1] * __builtin_amdgcn_exp2f(ms - m);
+  }
+  const float inv = 1.0f / l;
+  T* out = reinterpret_cast<T*>(p.out) + (int64_t)unit * H;
+  for (int h = threadIdx.x; h < H; h += NT) {
+    float o = 0.f;
+    for (int s = 0; s < p.splits; ++s) {
+      const float ms = wsu[(int64_t)s * (H + 2) + H];
+      if (ms > -INFINITY) o += wsu[(int64_t)s * (H + 2) + h] * __builtin_amdgcn_exp2f(ms - m);
+    }
+    out[h] = (T)(o * inv);
+  }
+}
+
+void plan(uint32_t units, uint32_t T, int* splits, int* chunk) {
+  // About 1024 work-groups in flight, at least 64 and at most 512 keys per chunk.
+  int s = (int)((1024 + units - 1) / units);
+  int c = (int)((T + s - 1) / s);
+  if (c < 64) c = 64;
+  if (c > 512) c = 512;
+  c = (c + 31) / 32 * 32;
+  *chunk = c;
+  *splits = (int)((T + c - 1) / c);
+}
+
+template <typename T>
+void launch(const DecodeParams& p, int units, hipStream_t st) {
+  const dim3 grid((unsigned)(units * p.splits)), block(NT);
+  if (p.H <= 64) hipLaunchKernelGGL((fmha_decode_split_kernel<T, 8>), grid, block, 0, st, p);
+  else if (p.H <= 128) hipLaunchKernelGGL((fmha_decode_split_kernel<T, 16>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((fmha_decode_split_kernel<T, 32>), grid, block, 0, st, p);
+  hipLaunchKernelGGL((fmha_decode_merge_kernel<T>), dim3((unsigned)units), block, 0, st, p);
+}
+
+}  // namespace
+
+extern "C" size_t xmk_fmha_decode_workspace_bytes(uint32_t num_batches, uint32_t num_heads,
+                                                  uint32_t head_size, uint32_t num_keys) {
+  int splits, chunk;
+  const uint32_t units = num_batches * num_heads;
+  if (units == 0 || num_keys == 0) return 0;
+  plan(units, num_keys, &splits, &chunk);
+  return (size_t)units * splits * (head_size + 2) * sizeof(float);
+}
+
+extern "C" int xmk_fmha_decode(const void* query, const void* key, const void* value, void* out,
+                               int32_t dtype, uint32_t num_batches, uint32_t num_heads,
+                               uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
+                               float head_scale, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  if (!query || !key || !value || !out || !workspace)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: null pointer");
+  if (dtype != XMK_F16 && dtype != XMK_BF16) return xmk::fail(XMK_INTERNAL, "Invalid MHA datatype");
+  if (num_batches == 0 || num_heads == 0 || head_size == 0 || num_keys == 0)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: empty dimension");
+  if (head_size > 256 || head_size % 8 != 0)
+    return xmk::fail(XMK_UNIMPLEMENTED, "fmha_decode: head_size must be a multiple of 8, at most 256");
+  if (kv_head_stride < (int64_t)num_keys * head_size || kv_head_stride % 8 != 0)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: kv_head_stride too small or not a multiple of 8");
+  if (!xmk::aligned(query, 16) || !xmk::aligned(key, 16) || !xmk::aligned(value, 16))
+    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: tensors must be 16-byte aligned");
+  const size_t need = xmk_fmha_decode_workspace_bytes(num_batches, num_heads, head_size, num_keys);
+  if (workspace_bytes < need)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+  DecodeParams p;
+  p.q = query; p.k = key; p.v = value; p.out = out; p.ws = (float*)workspace;
+  p.N = (int)num_heads; p.H = (int)head_size; p.T = (int)num_keys;
+  p.kv_head_stride = kv_head_stride;
+  p.scale2 = head_scale * kLog2e;
+  const uint32_t units = num_batches * num_heads;
+  plan(units, num_keys, &p.splits, &p.chunk);
+  xmk::trace("fmha_decode B=%u N=%u T=%u H=%u splits=%d chunk=%d", num_batches, num_heads, num_keys,
+             head_size, p.splits, p.chunk);
+  if (dtype == XMK_BF16) launch<__bf16>(p, (int)units, (hipStream_t)stream);
+  else launch<_Float16>(p, (int)units, (hipStream_t)stream);
+  return xmk::check_launch("fmha_decode");
+}

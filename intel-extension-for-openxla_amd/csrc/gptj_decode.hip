@@ -1,0 +1,197 @@
+// GPT-J-shaped decode step on int4 weights: the glue kernels (LayerNorm, rotary embedding
+// fused with the KV-cache append) and the host loop that strings them together with the
+// int4 GEMM and the split-key decode attention.  Everything is enqueued on one stream, in
+// order, with no host synchronisation, so a caller can capture the whole step in a HIP graph.
+#include "common.h"
+#include "int4_gemm.h"
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// y = (x - mean) / sqrt(var + eps) * gamma + beta, one work-group per row, fp32 statistics.
+__global__ __launch_bounds__(256) void layernorm_kernel(const _Float16* __restrict__ x,
+                                                        const _Float16* __restrict__ gamma,
+                                                        const _Float16* __restrict__ beta,
+                                                        _Float16* __restrict__ y, int d, float eps) {
+  __shared__ float s_part[2][4];
+  const _Float16* xr = x + (size_t)blockIdx.x * d;
+  float s = 0.f, ss = 0.f;
+  for (int i = threadIdx.x; i < d; i += 256) {
+    const float v = (float)xr[i];
+    s += v;
+    ss += v * v;
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    s += __shfl_xor(s, o);
+    ss += __shfl_xor(ss, o);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_part[0][threadIdx.x >> 6] = s;
+    s_part[1][threadIdx.x >> 6] = ss;
+  }
+  __syncthreads();
+  s = s_part[0][0] + s_part[0][1] + s_part[0][2] + s_part[0][3];
+  ss = s_part[1][0] + s_part[1][1] + s_part[1][2] + s_part[1][3];
+  const float mean = s / d;
+  const float var = fmaxf(ss / d - mean * mean, 0.f);
+  const float rstd = rsqrtf(var + eps);
+  for (int i = threadIdx.x; i < d; i += 256)
+    y[(size_t)blockIdx.x * d + i] = (_Float16)(((float)xr[i] - mean) * rstd * (float)gamma[i] + (float)beta[i]);
+}
+
+// qkv [B, 3 d] (columns q | k | v, head-major).  Rotates the first rotary_dim dims of every q
+// and k head (interleaved pairs, angle = position * 10000^(-2i/rotary_dim)); writes q to
+// q_out [B, d], and k (rotated) and v to row `position` of the caches [B, N, cap, H].
+__global__ __launch_bounds__(256) void rope_append_kernel(const _Float16* __restrict__ qkv,
+                                                          _Float16* __restrict__ q_out,
+                                                          _Float16* __restrict__ k_cache,
+                                                          _Float16* __restrict__ v_cache, int n_head,
+                                                          int head_dim, int rotary_dim, int cap,
+                                                          int position) {
+  const int b = blockIdx.y, head = blockIdx.x;
+  const int d = n_head * head_dim;
+  const _Float16* q = qkv + (size_t)b * 3 * d + (size_t)head * head_dim;
+  const _Float16* k = q + d;
+  const _Float16* v = q + 2 * d;
+  _Float16* qo = q_out + (size_t)b * d + (size_t)head * head_dim;
+  const size_t crow = (((size_t)b * n_head + head) * cap + position) * head_dim;
+  for (int i = threadIdx.x; i < head_dim / 2; i += 256) {
+    float q0 = (float)q[2 * i], q1 = (float)q[2 * i + 1];
+    float k0 = (float)k[2 * i], k1 = (float)k[2 * i + 1];
+    if (2 * i < rotary_dim) {
+      const float inv_freq = powf(10000.0f, -(float)(2 * i) / (float)rotary_dim);
+      float sn, cs;
+      sincosf((float)position * inv_freq, &sn, &cs);
+      const float a = q0 * cs - q1 * sn, bq = q1 * cs + q0 * sn;
+      q0 = a; q1 = bq;
+      const float c = k0 * cs - k1 * sn, dk = k1 * cs + k0 * sn;
+      k0 = c; k1 = dk;
+    }
+    qo[2 * i] = (_Float16)q0;
+    qo[2 * i + 1] = (_Float16)q1;
+    k_cache[crow + 2 * i] = (_Float16)k0;
+    k_cache[crow + 2 * i + 1] = (_Float16)k1;
+    v_cache[crow + 2 * i] = v[2 * i];
+    v_cache[crow + 2 * i + 1] = v[2 * i + 1];
+  }
+}
+
+struct Workspace {
+  _Float16 *x0, *x1, *h, *qkv, *q, *attn, *ff;
+  void* attn_ws;
+  size_t attn_ws_bytes;
+  size_t total;
+};
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+Workspace carve(const xmk_gptj_config& c, char* base) {
+  Workspace w;
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    char* p = base ? base + off : nullptr;
+    off += align_up(bytes);
+    return p;
+  };
+  const size_t B = (size_t)c.batch, d = (size_t)c.d_model;
+  w.x0 = (_Float16*)take(B * d * 2);
+  w.x1 = (_Float16*)take(B * d * 2);
+  w.h = (_Float16*)take(B * d * 2);
+  w.qkv = (_Float16*)take(B * 3 * d * 2);
+  w.q = (_Float16*)take(B * d * 2);
+  w.attn = (_Float16*)take(B * d * 2);
+  w.ff = (_Float16*)take(B * (size_t)c.d_ff * 2);
+  w.attn_ws_bytes = xmk_fmha_decode_workspace_bytes((uint32_t)c.batch, (uint32_t)c.n_head,
+                                                    (uint32_t)c.head_dim, (uint32_t)c.cache_capacity);
+  w.attn_ws = take(w.attn_ws_bytes);
+  w.total = off;
+  return w;
+}
+
+int check_cfg(const xmk_gptj_config* c) {
+  if (!c) return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: null config");
+  if (c->n_layer < 1 || c->n_head < 1 || c->head_dim < 8 || c->batch < 1 || c->cache_capacity < 1 ||
+      c->d_ff < 1 || c->vocab < 1)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: non-positive dimension");
+  if (c->d_model != c->n_head * c->head_dim)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: d_model != n_head * head_dim");
+  if (c->head_dim % 8 != 0 || c->head_dim > 256 || c->rotary_dim % 2 != 0 || c->rotary_dim > c->head_dim)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: unsupported head_dim / rotary_dim");
+  return XMK_OK;
+}
+
+int linear(const xmk_int4_linear& l, const void* act, void* out, int64_t m, int64_t k, int64_t n,
+           int64_t group, const xmk::Int4Epilogue& ep, hipStream_t st, const char* what) {
+  if (l.k != k || l.n != n)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: %s is %lldx%lld, expected %lldx%lld", what,
+                     (long long)l.k, (long long)l.n, (long long)k, (long long)n);
+  return xmk::int4_gemm_launch(act, l.qweight, l.scales, l.zeros, l.bias, out, m, k, n, group, ep, st);
+}
+
+}  // namespace
+
+extern "C" size_t xmk_gptj_decode_workspace_bytes(const xmk_gptj_config* cfg) {
+  if (check_cfg(cfg) != XMK_OK) return 0;
+  return carve(*cfg, nullptr).total;
+}
+
+extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_layer* layers,
+                                    const void* lnf_gamma, const void* lnf_beta,
+                                    const xmk_int4_linear* lm_head, const void* hidden_in,
+                                    int32_t position, void* logits, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  int rc = check_cfg(cfg);
+  if (rc != XMK_OK) return rc;
+  if (!layers || !lnf_gamma || !lnf_beta || !lm_head || !hidden_in || !logits || !workspace)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: null pointer");
+  if (position < 0 || position >= cfg->cache_capacity)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: position %d outside the cache (capacity %d)",
+                     position, cfg->cache_capacity);
+  if (!xmk::aligned(workspace, 256)) return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: workspace must be 256-byte aligned");
+  const xmk_gptj_config& c = *cfg;
+  const Workspace w = carve(c, (char*)workspace);
+  if (workspace_bytes < w.total)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: workspace of %zu bytes, %zu needed", workspace_bytes, w.total);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t B = c.batch, d = c.d_model, dff = c.d_ff;
+  const float scale = 1.0f / sqrtf((float)c.head_dim);
+  const int64_t head_stride = (int64_t)c.cache_capacity * c.head_dim;
+
+  const _Float16* x = (const _Float16*)hidden_in;
+  _Float16* xn = w.x0;
+  for (int l = 0; l < c.n_layer; ++l) {
+    const xmk_gptj_layer& L = layers[l];
+    if (!L.ln_gamma || !L.ln_beta || !L.k_cache || !L.v_cache)
+      return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: layer %d has a null pointer", l);
+    hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(256), 0, st, x, (const _Float16*)L.ln_gamma,
+                       (const _Float16*)L.ln_beta, w.h, (int)d, c.ln_eps);
+    if ((rc = linear(L.qkv, w.h, w.qkv, B, d, 3 * d, c.group, xmk::Int4Epilogue{}, st, "qkv")) != XMK_OK) return rc;
+    hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)c.n_head, (unsigned)B), dim3(256), 0, st, w.qkv, w.q,
+                       (_Float16*)L.k_cache, (_Float16*)L.v_cache, c.n_head, c.head_dim, c.rotary_dim,
+                       c.cache_capacity, position);
+    if ((rc = xmk_fmha_decode(w.q, L.k_cache, L.v_cache, w.attn, XMK_F16, (uint32_t)B, (uint32_t)c.n_head,
+                              (uint32_t)c.head_dim, (uint32_t)(position + 1), head_stride, scale, w.attn_ws,
+                              w.attn_ws_bytes, stream)) != XMK_OK)
+      return rc;
+    // fc_in (+bias, gelu_new) from the same ln_1 output; fc_out adds bias, the residual x and the
+    // attention branch in its epilogue:  x' = x + out_proj(attn) + fc_out(...)
+    xmk::Int4Epilogue gelu;
+    gelu.gelu = 1;
+    if ((rc = linear(L.fc_in, w.h, w.ff, B, d, dff, c.group, gelu, st, "fc_in")) != XMK_OK) return rc;
+    // out_proj result goes to w.qkv's first B*d elements (qkv is dead after the rotary kernel)
+    _Float16* a_out = w.qkv;
+    if ((rc = linear(L.out_proj, w.attn, a_out, B, d, d, c.group, xmk::Int4Epilogue{}, st, "out_proj")) != XMK_OK) return rc;
+    xmk::Int4Epilogue res;
+    res.add0 = x;
+    res.add1 = a_out;
+    if ((rc = linear(L.fc_out, w.ff, xn, B, dff, d, c.group, res, st, "fc_out")) != XMK_OK) return rc;
+    x = xn;
+    xn = (xn == w.x0) ? w.x1 : w.x0;
+  }
+  hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(256), 0, st, x, (const _Float16*)lnf_gamma,
+                     (const _Float16*)lnf_beta, w.h, (int)d, c.ln_eps);
+  if ((rc = linear(*lm_head, w.h, logits, B, d, c.vocab, c.group, xmk::Int4Epilogue{}, st, "lm_head")) != XMK_OK) return rc;
+  return xmk::check_launch("gptj_decode");
+}

@@ -10,6 +10,7 @@
 //     out[m,n] = sum_g s[g,n] * ( sum_{k in g} a[m,k] q[k,n]  -  z[g,n] * sum_{k in g} a[m,k] )
 // where the second sum comes from one extra MFMA against a B operand of ones.
 #include "common.h"
+#include "int4_gemm.h"
 
 namespace {
 
@@ -82,7 +83,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
     const _Float16* __restrict__ act, const uint32_t* __restrict__ qw,
     const _Float16* __restrict__ scales, const _Float16* __restrict__ zeros,
     const _Float16* __restrict__ bias, _Float16* __restrict__ out, int m_base, int M, int K,
-    int N) {
+    int N, xmk::Int4Epilogue ep) {
   constexpr int NCOL = 16 * W;
   __shared__ float red[NW][MT * 16][NCOL];
 
@@ -192,7 +193,14 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
 #pragma unroll
     for (int w = 0; w < NW; ++w) s += red[w][row][col];
     if (bias) s += (float)bias[n];
-    out[(size_t)(m_base + row) * N + n] = (_Float16)s;
+    if (ep.gelu) {  // gelu_new: 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) = x / (1 + e^{-2u})
+      const float u = 0.7978845608028654f * (s + 0.044715f * s * s * s);
+      s = s / (1.0f + __expf(-2.0f * u));
+    }
+    const size_t o = (size_t)(m_base + row) * N + n;
+    if (ep.add0) s += (float)reinterpret_cast<const _Float16*>(ep.add0)[o];
+    if (ep.add1) s += (float)reinterpret_cast<const _Float16*>(ep.add1)[o];
+    out[o] = (_Float16)s;
   }
 }
 
@@ -229,21 +237,23 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(
 
 template <int W, int MT, int SPG, int NW>
 void launch(const void* act, const void* qw, const void* scales, const void* zeros,
-            const void* bias, void* out, int m_base, int M, int K, int N, hipStream_t st) {
+            const void* bias, void* out, int m_base, int M, int K, int N,
+            const xmk::Int4Epilogue& ep, hipStream_t st) {
   const int blocks = (int)xmk::ceil_div(N, 16 * W);
   hipLaunchKernelGGL((int4_gemm_kernel<W, MT, SPG, NW>), dim3(blocks), dim3(NW * 64), 0, st,
                      (const _Float16*)act, (const uint32_t*)qw, (const _Float16*)scales,
-                     (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N);
+                     (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N, ep);
 }
 
 template <int W, int MT, int NW>
 int launch_spg(int spg, const void* act, const void* qw, const void* scales, const void* zeros,
-               const void* bias, void* out, int m_base, int M, int K, int N, hipStream_t st) {
+               const void* bias, void* out, int m_base, int M, int K, int N,
+               const xmk::Int4Epilogue& ep, hipStream_t st) {
   switch (spg) {
-    case 1: launch<W, MT, 1, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, st); break;
-    case 2: launch<W, MT, 2, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, st); break;
-    case 4: launch<W, MT, 4, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, st); break;
-    case 8: launch<W, MT, 8, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, st); break;
+    case 1: launch<W, MT, 1, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 2: launch<W, MT, 2, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 4: launch<W, MT, 4, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 8: launch<W, MT, 8, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
     default: return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   }
   return XMK_OK;
@@ -251,9 +261,9 @@ int launch_spg(int spg, const void* act, const void* qw, const void* scales, con
 
 }  // namespace
 
-extern "C" int xmk_int4_gemm(const void* act, const void* qweight, const void* scales,
-                             const void* zeros, const void* bias, void* out, int64_t m, int64_t k,
-                             int64_t n, int64_t group, void* stream) {
+int xmk::int4_gemm_launch(const void* act, const void* qweight, const void* scales,
+                          const void* zeros, const void* bias, void* out, int64_t m, int64_t k,
+                          int64_t n, int64_t group, const Int4Epilogue& ep, hipStream_t st) {
   if (!act || !qweight || !scales || !zeros || !out)
     return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: null pointer");
   if (m <= 0 || k <= 0 || n <= 0 || group <= 0)
@@ -269,7 +279,6 @@ extern "C" int xmk_int4_gemm(const void* act, const void* qweight, const void* s
   if (!xmk::aligned(act, 16) || !xmk::aligned(qweight, 16) || !xmk::aligned(scales, 2) ||
       !xmk::aligned(out, 2))
     return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: act and qweight must be 16-byte aligned");
-  hipStream_t st = (hipStream_t)stream;
   const int spg = (int)(group / 32);
   const int M = (int)m, K = (int)k, N = (int)n;
   // Words per lane: the widest load that still yields about one block per CU.
@@ -280,9 +289,9 @@ extern "C" int xmk_int4_gemm(const void* act, const void* qweight, const void* s
   for (int m_base = 0; m_base < M; m_base += 32) {
     const bool two = (M - m_base) > 16;
     int rc;
-#define XMK_INT4_CASE(WW)                                                                        \
-  rc = two ? launch_spg<WW, 2, 8>(spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, st) \
-           : launch_spg<WW, 1, 16>(spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, st)
+#define XMK_INT4_CASE(WW)                                                                            \
+  rc = two ? launch_spg<WW, 2, 8>(spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st) \
+           : launch_spg<WW, 1, 16>(spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st)
     if (w == 4) { XMK_INT4_CASE(4); }
     else if (w == 2) { XMK_INT4_CASE(2); }
     else { XMK_INT4_CASE(1); }
@@ -290,6 +299,13 @@ extern "C" int xmk_int4_gemm(const void* act, const void* qweight, const void* s
     if (rc != XMK_OK) return rc;
   }
   return xmk::check_launch("int4_gemm");
+}
+
+extern "C" int xmk_int4_gemm(const void* act, const void* qweight, const void* scales,
+                             const void* zeros, const void* bias, void* out, int64_t m, int64_t k,
+                             int64_t n, int64_t group, void* stream) {
+  return xmk::int4_gemm_launch(act, qweight, scales, zeros, bias, out, m, k, n, group,
+                               xmk::Int4Epilogue{}, (hipStream_t)stream);
 }
 
 extern "C" int xmk_int4_dequant(const void* qweight, const void* scales, const void* zeros,
