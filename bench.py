@@ -81,6 +81,18 @@ def wl_gemm(torch, xmk, m, n, k, bias=False, rhs_t=False):
                 bound="mfma", dtype="bf16", kernel="gemm_mfma_kernel")
 
 
+def wl_fp8(torch, xmk, m, n, k):
+    a = torch.randn((m, k), device="cuda")
+    b = torch.randn((n, k), device="cuda")
+    sa, sb = a.abs().max() / 448.0, b.abs().max() / 448.0
+    qa, qb = (a / sa).to(torch.float8_e4m3fn), (b / sb).to(torch.float8_e4m3fn)
+    sa, sb = sa.reshape(1).float(), sb.reshape(1).float()
+    out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    return dict(name=f"gemm_fp8_e4m3_{m}x{n}x{k}_rhsT", fn=lambda: xmk.fp8_gemm(qa, qb, sa, sb, out, rhs_transpose=True),
+                flops=2.0 * m * n * k, bytes=1.0 * (m * k + k * n) + 2.0 * m * n, bound="mfma", dtype="fp8",
+                kernel="fp8_gemm_kernel")
+
+
 def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
     # Rotate through `copies` weight sets (12 x 35.7 MB > the 256 MB last-level cache) so that
     # every launch streams its weights from HBM.
@@ -101,6 +113,40 @@ def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
                 bound="hbm", dtype="f16", kernel="int4_gemm_kernel", graph=True)
 
 
+def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
+    """BASELINE config 5: GPT-J-6B-shaped decode step, int4 group-128 weights, fp16 KV cache filled to
+    `cache_len`, one new token per sequence.  The whole step (about 8 launches per block) is replayed
+    from one HIP graph."""
+    d, heads, hd, dff, vocab, g = 4096, 16, 256, 16384, 50400, 128
+    cap = cache_len + 1
+
+    def lin(k, n, bias):
+        qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 8, n), dtype=torch.int32, device="cuda")
+        sc = (torch.rand((k // g, n), device="cuda") * 0.019 + 0.001).half()
+        zp = (torch.rand((k // g, n), device="cuda") * 15).half()
+        b = (torch.randn((n,), device="cuda") * 0.02).half() if bias else None
+        return qw, sc, zp, b
+
+    layers = []
+    for _ in range(n_layer):
+        layers.append(dict(ln_gamma=torch.ones((d,), device="cuda").half(), ln_beta=torch.zeros((d,), device="cuda").half(),
+                           qkv=lin(d, 3 * d, False), out_proj=lin(d, d, False), fc_in=lin(d, dff, True),
+                           fc_out=lin(dff, d, True),
+                           k_cache=torch.randn((batch, heads, cap, hd), device="cuda").half(),
+                           v_cache=torch.randn((batch, heads, cap, hd), device="cuda").half()))
+    cfg = xmk.GptjConfig(n_layer, heads, hd, 64, d, dff, vocab, g, batch, cap, 1e-5)
+    dec = xmk.GptjDecoder(cfg, layers, torch.ones((d,), device="cuda").half(), torch.zeros((d,), device="cuda").half(),
+                          lin(d, vocab, True))
+    hidden = torch.randn((batch, d), device="cuda").half()
+    logits = torch.empty((batch, vocab), dtype=torch.float16, device="cuda")
+    wbytes = n_layer * ((4 * d * d + 2 * d * dff) / 2 + (4 * d * d + 2 * d * dff) / g * 4) \
+        + d * vocab / 2 + d * vocab / g * 4
+    kvbytes = n_layer * 2.0 * batch * heads * cap * hd * 2
+    return dict(name=f"gptj6b_decode_step_int4_l{n_layer}_b{batch}_kv{cache_len}", fn=lambda: dec.step(hidden, cache_len, logits),
+                flops=0.0, bytes=wbytes + kvbytes, bound="hbm", dtype="f16", kernel="int4_gemm_kernel + fmha_decode_split_kernel",
+                graph=True, graph_steps=3)
+
+
 WORKLOADS = {
     "fmha_causal": lambda t, x: wl_fmha(t, x, True),
     "fmha": lambda t, x: wl_fmha(t, x, False),
@@ -110,15 +156,19 @@ WORKLOADS = {
     "int4_m1": lambda t, x: wl_int4(t, x, 1),
     "int4_m8": lambda t, x: wl_int4(t, x, 8),
     "int4_m32": lambda t, x: wl_int4(t, x, 32),
+    "fp8_8192": lambda t, x: wl_fp8(t, x, 8192, 8192, 8192),
+    "gptj_decode": lambda t, x: wl_gptj_decode(t, x),
 }
-ALSO = ["gemm_8192", "gemm_c1", "int4_m1", "int4_m8", "int4_m32"]
+ALSO = ["gemm_8192", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "gptj_decode"]
 
 
 def measure(torch, xmk, key, steps, warmup):
     w = WORKLOADS[key](torch, xmk)
+    if "graph_steps" in w:
+        steps, warmup = min(steps, w["graph_steps"]), min(warmup, 1)
     ms, wall_ms = _events(torch, w["fn"], steps, warmup, graph=w.get("graph", False))
     if w["bound"] == "mfma":
-        achieved, peak, unit = w["flops"] / ms / 1e9, PEAK["bf16"], "TFLOP/s"
+        achieved, peak, unit = w["flops"] / ms / 1e9, PEAK["fp8" if w["dtype"] == "fp8" else "bf16"], "TFLOP/s"
     else:
         achieved, peak, unit = w["bytes"] / ms / 1e6, HBM_PEAK, "GB/s"
     roof = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
