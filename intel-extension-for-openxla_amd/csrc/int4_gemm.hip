@@ -8,7 +8,11 @@
 // core; nothing is staged through LDS.  Zero points and scales are applied once
 // per quantisation group on the fp32 accumulator:
 //     out[m,n] = sum_g s[g,n] * ( sum_{k in g} a[m,k] q[k,n]  -  z[g,n] * sum_{k in g} a[m,k] )
-// where the second sum comes from one extra MFMA against a B operand of ones.
+// where the second sum comes from one extra MFMA against a B operand of ones.  The kernel
+// is bound by HBM only if the per-weight VALU work stays near one operation, so the
+// nibbles are expanded with the fp16 "magic number" trick (5 operations per 8 weights).
+#include <cstdlib>
+
 #include "common.h"
 #include "int4_gemm.h"
 
@@ -25,21 +29,27 @@ union Frag {
   half2v p[4];
 };
 
-// One packed word -> 8 exact fp16 integers, in k-slot order (0,4,1,5,2,6,3,7).
-// 0x6400 | q is 1024 + q; 0x5400 | (q << 4) is 64 + q; the packed subtract is exact.
-__device__ __forceinline__ half8 unpack_word(uint32_t w) {
+// (a & mask) | magic.  `magic_vgpr` must be a value the compiler cannot see through (it is
+// laundered through an empty asm at the call site): with a known constant it emits separate
+// v_and and v_or (VOP3 takes one scalar source and no literal), with an opaque VGPR it selects
+// the single v_and_or_b32.  No instruction is written by hand here on purpose: the hazard
+// recogniser cannot see inside inline asm, and these results feed MFMAs.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t magic_vgpr) {
+  return (a & mask) | magic_vgpr;
+}
+
+// One packed word -> 8 fp16 values q + offset, in k-slot order (0,4,1,5,2,6,3,7):
+// 0x6400 | q is 1024 + q (slots 0,1,4,5) and 0x5400 | (q << 4) is 64 + q (slots 2,3,6,7).
+// The offsets are not subtracted here (that would cost as many VALU operations again);
+// they are removed per quantisation group through sum_k a_k * offset_k, which one extra
+// MFMA against a constant fragment provides.  5 VALU operations per 8 weights.
+__device__ __forceinline__ half8 unpack_word(uint32_t w, uint32_t m1024, uint32_t m64) {
   const uint32_t w8 = w >> 8;
   Frag f;
-  f.u[0] = (w & 0x000f000fu) | 0x64006400u;
-  f.u[1] = (w & 0x00f000f0u) | 0x54005400u;
-  f.u[2] = (w8 & 0x000f000fu) | 0x64006400u;
-  f.u[3] = (w8 & 0x00f000f0u) | 0x54005400u;
-  const half2v k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
-  const half2v k64 = {(_Float16)64.0f, (_Float16)64.0f};
-  f.p[0] -= k1024;
-  f.p[1] -= k64;
-  f.p[2] -= k1024;
-  f.p[3] -= k64;
+  f.u[0] = and_or(w, 0x000f000fu, m1024);
+  f.u[1] = and_or(w, 0x00f000f0u, m64);
+  f.u[2] = and_or(w8, 0x000f000fu, m1024);
+  f.u[3] = and_or(w8, 0x00f000f0u, m64);
   return f.h;
 }
 
@@ -53,56 +63,86 @@ __device__ __forceinline__ half8 permute_act(u32x4 d) {
   return f.h;
 }
 
-template <int W>
+constexpr uint32_t kOob = 0x80000000u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+template <int NWORDS>
 struct Words {
-  uint32_t w[W];
+  uint32_t w[NWORDS];
 };
 
-template <int W>
-__device__ __forceinline__ Words<W> load_words(const uint32_t* p) {
-  Words<W> r;
-  if constexpr (W == 4) {
-    u32x4 v = *reinterpret_cast<const u32x4*>(p);
-    r.w[0] = v[0]; r.w[1] = v[1]; r.w[2] = v[2]; r.w[3] = v[3];
-  } else if constexpr (W == 2) {
-    uint2 v = *reinterpret_cast<const uint2*>(p);
-    r.w[0] = v.x; r.w[1] = v.y;
+// NWORDS consecutive dwords at byte offset voff + soff of a buffer.
+template <int NWORDS>
+__device__ __forceinline__ Words<NWORDS> load_words(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  Words<NWORDS> o;
+  if constexpr (NWORDS == 4) {
+    const u32x4 v = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+    o.w[0] = v[0]; o.w[1] = v[1]; o.w[2] = v[2]; o.w[3] = v[3];
+  } else if constexpr (NWORDS == 2) {
+    const auto v = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0);
+    o.w[0] = v[0]; o.w[1] = v[1];
   } else {
-    r.w[0] = *p;
+    o.w[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
   }
-  return r;
+  return o;
+}
+// W consecutive fp16 values at byte offset voff + soff, as packed dwords.
+template <int W>
+__device__ __forceinline__ Words<(W + 1) / 2> load_halves(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  if constexpr (W == 1) {
+    Words<1> o;
+    o.w[0] = __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+    return o;
+  } else {
+    return load_words<W / 2>(r, voff, soff);
+  }
+}
+template <int NWORDS>
+__device__ __forceinline__ float half_at(const Words<NWORDS>& r, int c) {
+  const uint16_t bits = (uint16_t)(r.w[c / 2] >> (16 * (c % 2)));
+  return (float)__builtin_bit_cast(_Float16, bits);
 }
 
 // W    : words (output channels) per lane; a block covers 16*W output channels
 // MT   : 16-row activation tiles (1 or 2)
+// RI   : accumulator rows per lane that can be live (4, or fewer when M <= 4 so that the
+//        per-group fix-up only touches rows that exist)
 // SPG  : 32-channel k-steps per quantisation group (group = 32*SPG)
 // NW   : waves per block; wave w takes groups w, w+NW, ... and the partial
 //        sums meet in LDS in a fixed order (deterministic result)
-template <int W, int MT, int SPG, int NW>
+template <int W, int MT, int RI, int SPG, int NW>
 __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
     const _Float16* __restrict__ act, const uint32_t* __restrict__ qw,
     const _Float16* __restrict__ scales, const _Float16* __restrict__ zeros,
     const _Float16* __restrict__ bias, _Float16* __restrict__ out, int m_base, int M, int K,
     int N, xmk::Int4Epilogue ep) {
   constexpr int NCOL = 16 * W;
-  __shared__ float red[NW][MT * 16][NCOL];
+  constexpr int ROWS = MT == 2 ? 32 : (RI == 4 ? 16 : RI);  // rows the block reduces
+  __shared__ float red[NW][ROWS][NCOL];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
   const int kg = lane >> 4;
   const int n0 = blockIdx.x * NCOL + col16 * W;
   const bool col_ok = n0 < N;
-  const int nsafe = col_ok ? n0 : 0;
   const int ngroups = K / (32 * SPG);
 
-  const _Float16* arow[MT];
-  bool row_ok[MT];
+  // Buffer descriptors: hardware bounds checking zero-fills lanes that are out of range
+  // (offset kOob), and the per-lane byte offsets below never change inside the K loop.
+  const __amdgpu_buffer_rsrc_t r_w = make_rsrc(qw, (uint32_t)((size_t)(K / 8) * N * 4));
+  const __amdgpu_buffer_rsrc_t r_s = make_rsrc(scales, (uint32_t)((size_t)ngroups * N * 2));
+  const __amdgpu_buffer_rsrc_t r_z = make_rsrc(zeros, (uint32_t)((size_t)ngroups * N * 2));
+  const __amdgpu_buffer_rsrc_t r_a = make_rsrc(act + (size_t)m_base * K, (uint32_t)((size_t)(M - m_base) * K * 2));
+  const uint32_t voff_w = col_ok ? (uint32_t)((kg * N + n0) * 4) : kOob;
+  const uint32_t voff_sz = col_ok ? (uint32_t)(n0 * 2) : kOob;
+  uint32_t voff_a[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int m = m_base + mt * 16 + col16;
-    row_ok[mt] = m < M;
-    arow[mt] = act + (size_t)(row_ok[mt] ? m : 0) * K + 8 * kg;
+    const int m = mt * 16 + col16;
+    voff_a[mt] = (m_base + m < M) ? (uint32_t)((m * K + 8 * kg) * 2) : kOob;
   }
 
   floatx4 acc[MT][W];
@@ -111,80 +151,101 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
 #pragma unroll
     for (int c = 0; c < W; ++c) acc[mt][c] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  Frag ones;
+  Frag ones, offs;  // B operands that yield sum_k a_k and sum_k a_k * offset_k
 #pragma unroll
-  for (int i = 0; i < 4; ++i) ones.u[i] = 0x3c003c00u;
+  for (int i = 0; i < 4; ++i) {
+    ones.u[i] = 0x3c003c00u;
+    offs.u[i] = (i & 1) ? 0x54005400u : 0x64006400u;
+  }
+  uint32_t m1024 = 0x64006400u, m64 = 0x54005400u;
+  asm volatile("" : "+v"(m1024), "+v"(m64));  // keep the magic constants in VGPRs
 
-  Words<W> cur[SPG], nxt[SPG];
-  int g = wave;
-  if (g < ngroups) {
+  // Everything a group needs (scales, zero points, activations, weights) is fetched one
+  // group ahead, weights last: vector loads return in order, so computing group g waits only
+  // for loads issued an iteration earlier, never for the prefetch of group g + NW.
+  struct GroupData {
+    Words<W> w[SPG];
+    Words<(W + 1) / 2> sc, zp;
+    u32x4 a[SPG][MT];
+  };
+  auto fetch = [&](int g, GroupData& d) {
+    const uint32_t so = (uint32_t)(g * N * 2);
+    d.sc = load_halves<W>(r_s, voff_sz, so);
+    d.zp = load_halves<W>(r_z, voff_sz, so);
 #pragma unroll
     for (int s = 0; s < SPG; ++s)
-      cur[s] = load_words<W>(qw + (size_t)(g * 4 * SPG + s * 4 + kg) * N + nsafe);
-  }
-  for (; g < ngroups; g += NW) {
-    const int gn = g + NW;
-    if (gn < ngroups) {
 #pragma unroll
-      for (int s = 0; s < SPG; ++s)
-        nxt[s] = load_words<W>(qw + (size_t)(gn * 4 * SPG + s * 4 + kg) * N + nsafe);
-    }
-    _Float16 sc[W], zp[W];
+      for (int mt = 0; mt < MT; ++mt)
+        d.a[s][mt] = __builtin_bit_cast(
+            u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_a, voff_a[mt], (uint32_t)((g * SPG + s) * 64), 0));
 #pragma unroll
-    for (int c = 0; c < W; ++c) {
-      sc[c] = scales[(size_t)g * N + nsafe + c];
-      zp[c] = zeros[(size_t)g * N + nsafe + c];
-    }
-    floatx4 d[MT][W], asum[MT];
+    for (int s = 0; s < SPG; ++s)
+      d.w[s] = load_words<W>(r_w, voff_w, (uint32_t)((g * 4 * SPG + s * 4) * N * 4));
+  };
+  auto compute = [&](const GroupData& cur) {
+    floatx4 d[MT][W], asum[MT], aoff[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       asum[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+      aoff[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < W; ++c) d[mt][c] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 #pragma unroll
     for (int s = 0; s < SPG; ++s) {
-      const int k0 = (g * SPG + s) * 32;
       half8 a[MT];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        u32x4 raw = {0u, 0u, 0u, 0u};
-        if (row_ok[mt]) raw = *reinterpret_cast<const u32x4*>(arow[mt] + k0);
-        a[mt] = permute_act(raw);
-      }
+      for (int mt = 0; mt < MT; ++mt) a[mt] = permute_act(cur.a[s][mt]);
 #pragma unroll
       for (int c = 0; c < W; ++c) {
-        const half8 b = unpack_word(cur[s].w[c]);
+        const half8 b = unpack_word(cur.w[s].w[c], m1024, m64);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
           d[mt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], b, d[mt][c], 0, 0, 0);
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int mt = 0; mt < MT; ++mt) {
         asum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], ones.h, asum[mt], 0, 0, 0);
+        aoff[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], offs.h, aoff[mt], 0, 0, 0);
+      }
     }
+    // acc += s * (sum a (q + off) - sum a off - z sum a), only for rows that can exist
 #pragma unroll
     for (int c = 0; c < W; ++c) {
-      const float s = (float)sc[c], z = (float)zp[c];
+      const float sc = half_at(cur.sc, c), z = half_at(cur.zp, c);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[mt][c][i] += s * (d[mt][c][i] - z * asum[mt][i]);
+        for (int i = 0; i < RI; ++i)
+          acc[mt][c][i] = fmaf(sc, d[mt][c][i] - fmaf(z, asum[mt][i], aoff[mt][i]), acc[mt][c][i]);
     }
-#pragma unroll
-    for (int s = 0; s < SPG; ++s) cur[s] = nxt[s];
+  };
+
+  GroupData bufA, bufB;  // ping-pong: no register copies between iterations
+  int g = wave;
+  if (g < ngroups) fetch(g, bufA);
+  while (g < ngroups) {
+    if (g + NW < ngroups) fetch(g + NW, bufB);
+    compute(bufA);
+    g += NW;
+    if (g >= ngroups) break;
+    if (g + NW < ngroups) fetch(g + NW, bufA);
+    compute(bufB);
+    g += NW;
   }
 
-  // Lane holds rows 4*kg+i of columns col16*W+c.
+  // Lane holds rows 4*kg+i (+16 mt) of columns col16*W+c.
+  if (RI == 4 || kg == 0) {
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < RI; ++i)
 #pragma unroll
-      for (int c = 0; c < W; ++c) red[wave][mt * 16 + 4 * kg + i][col16 * W + c] = acc[mt][c][i];
+        for (int c = 0; c < W; ++c) red[wave][mt * 16 + (RI == 4 ? 4 * kg : 0) + i][col16 * W + c] = acc[mt][c][i];
+  }
   __syncthreads();
 
-  const int rows = min(MT * 16, M - m_base);
+  const int rows = min(ROWS, M - m_base);
   for (int e = threadIdx.x; e < rows * NCOL; e += NW * 64) {
     const int row = e / NCOL, col = e % NCOL;
     const int n = blockIdx.x * NCOL + col;
@@ -235,25 +296,25 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(
   }
 }
 
-template <int W, int MT, int SPG, int NW>
+template <int W, int MT, int RI, int SPG, int NW>
 void launch(const void* act, const void* qw, const void* scales, const void* zeros,
             const void* bias, void* out, int m_base, int M, int K, int N,
             const xmk::Int4Epilogue& ep, hipStream_t st) {
   const int blocks = (int)xmk::ceil_div(N, 16 * W);
-  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, SPG, NW>), dim3(blocks), dim3(NW * 64), 0, st,
+  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW>), dim3(blocks), dim3(NW * 64), 0, st,
                      (const _Float16*)act, (const uint32_t*)qw, (const _Float16*)scales,
                      (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N, ep);
 }
 
-template <int W, int MT, int NW>
+template <int W, int MT, int RI, int NW>
 int launch_spg(int spg, const void* act, const void* qw, const void* scales, const void* zeros,
                const void* bias, void* out, int m_base, int M, int K, int N,
                const xmk::Int4Epilogue& ep, hipStream_t st) {
   switch (spg) {
-    case 1: launch<W, MT, 1, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
-    case 2: launch<W, MT, 2, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
-    case 4: launch<W, MT, 4, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
-    case 8: launch<W, MT, 8, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 1: launch<W, MT, RI, 1, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 2: launch<W, MT, RI, 2, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 4: launch<W, MT, RI, 4, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 8: launch<W, MT, RI, 8, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
     default: return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   }
   return XMK_OK;
@@ -276,26 +337,44 @@ int xmk::int4_gemm_launch(const void* act, const void* qweight, const void* scal
     return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   if (k > (1 << 24) || n > (1 << 24) || m > (1 << 24))
     return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: dimension too large");
-  if (!xmk::aligned(act, 16) || !xmk::aligned(qweight, 16) || !xmk::aligned(scales, 2) ||
+  if (!xmk::aligned(act, 16) || !xmk::aligned(qweight, 16) || !xmk::aligned(scales, 8) || !xmk::aligned(zeros, 8) ||
       !xmk::aligned(out, 2))
-    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: act and qweight must be 16-byte aligned");
+    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: act, qweight must be 16-byte and scales, zeros 8-byte aligned");
   const int spg = (int)(group / 32);
   const int M = (int)m, K = (int)k, N = (int)n;
   // Words per lane: the widest load that still yields about one block per CU.
   int w = 4;
   if (N / 64 < 192) w = 2;
   if (N / 32 < 192) w = 1;
-  xmk::trace("int4_gemm m=%d k=%d n=%d group=%d words_per_lane=%d", M, K, N, (int)group, w);
+  int nw = 16;
+  // XMK_INT4_TILE="<words per lane>,<waves per block>" overrides the choice (tuning aid).
+  static const char* tile_env = getenv("XMK_INT4_TILE");
+  if (tile_env) {
+    int ew = 0, enw = 0;
+    if (sscanf(tile_env, "%d,%d", &ew, &enw) == 2 && (ew == 1 || ew == 2 || ew == 4) && (enw == 8 || enw == 16)) {
+      w = ew;
+      nw = enw;
+    }
+  }
+  xmk::trace("int4_gemm m=%d k=%d n=%d group=%d words_per_lane=%d waves=%d", M, K, N, (int)group, w, nw);
   for (int m_base = 0; m_base < M; m_base += 32) {
-    const bool two = (M - m_base) > 16;
+    const int rows = M - m_base;
     int rc;
-#define XMK_INT4_CASE(WW)                                                                            \
-  rc = two ? launch_spg<WW, 2, 8>(spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st) \
-           : launch_spg<WW, 1, 16>(spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st)
-    if (w == 4) { XMK_INT4_CASE(4); }
-    else if (w == 2) { XMK_INT4_CASE(2); }
-    else { XMK_INT4_CASE(1); }
+#define XMK_INT4_ARGS spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st
+#define XMK_INT4_CASE(WW)                                                   \
+  do {                                                                      \
+    if (rows > 16) rc = launch_spg<WW, 2, 4, 8>(XMK_INT4_ARGS);             \
+    else if (rows > 4) rc = launch_spg<WW, 1, 4, 8>(XMK_INT4_ARGS);         \
+    else if (rows > 1) rc = nw == 16 ? launch_spg<WW, 1, 4, 16>(XMK_INT4_ARGS) \
+                                     : launch_spg<WW, 1, 4, 8>(XMK_INT4_ARGS); \
+    else rc = nw == 16 ? launch_spg<WW, 1, 1, 16>(XMK_INT4_ARGS)            \
+                       : launch_spg<WW, 1, 1, 8>(XMK_INT4_ARGS);            \
+  } while (0)
+    if (w == 4) XMK_INT4_CASE(4);
+    else if (w == 2) XMK_INT4_CASE(2);
+    else XMK_INT4_CASE(1);
 #undef XMK_INT4_CASE
+#undef XMK_INT4_ARGS
     if (rc != XMK_OK) return rc;
   }
   return xmk::check_launch("int4_gemm");
