@@ -15,7 +15,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libxmk.so")
+LIB_PATH = os.environ.get("XMK_LIB") or os.path.join(_HERE, "libxmk.so")  # XMK_LIB: load another build
 
 # xla::PrimitiveType numbering
 S8, S32, F16, F32, BF16, F8E4M3FN = 2, 4, 10, 11, 16, 20

@@ -19,7 +19,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I", INCLUDE, "-I", CSRC,
          # packed-fp32 VALU forms are kept out of generated code on purpose
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes"]
+         "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes"] + os.environ.get("XMK_CXXFLAGS", "").split()
 
 
 def sources():
