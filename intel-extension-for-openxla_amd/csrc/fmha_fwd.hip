@@ -1,20 +1,25 @@
 // Fused multi-head attention forward (flash attention) for bf16 / fp16:
 //     O = softmax(scale * Q K^T + bias + mask) V,   optional LSE = m + log l.
 //
-// One work-group = 128 query rows of one (batch, head) unit, 4 waves x 32 rows.  Keys
-// are walked in blocks of 64.  Both products are issued transposed so that a lane owns
-// ONE query row for the whole kernel:
-//   S^T = K Q^T : A operand = K fragment (rows = keys), B operand = Q fragment kept in
-//                 registers; the 32x32 accumulator layout puts query l%32 in lane l and
-//                 keys in the lane's registers, so row max / row sum are plain register
-//                 reductions plus one exchange with lane l^32 (which holds the other keys).
-//   O^T += V^T P^T : P stays in registers (the accumulator registers, converted, ARE
-//                 the B operand); V is staged untransposed [key][h] and read with the LDS
-//                 transpose loads, which deliver four consecutive keys of one h.
-// Online softmax in the exp2 domain (scale * log2 e folded into one multiply), running
-// max m and per-lane partial sum l; O is rescaled by 2^(m_old - m_new) per block and
-// divided by l once at the end.  Causal: key > query masked (top-left aligned), key
-// blocks past the diagonal are never visited, work-groups are issued heaviest first.
+// One work-group = NW waves, each owning QT tiles of 32 query rows of one (batch, head)
+// unit; keys are walked in blocks of 64.  Both products are issued transposed so that a
+// lane owns ONE query row per tile for the whole kernel:
+//   S^T = K Q^T : A operand = K fragment (rows = keys) read from LDS, B operand = Q fragment
+//                 kept in registers; the 32x32 accumulator layout puts query l%32 in lane l
+//                 and keys in the lane's registers, so the row max is a register reduction
+//                 plus one exchange with lane l^32 (which holds the other keys).  A K fragment
+//                 read once from LDS feeds the MFMAs of all QT query tiles.
+//   O^T += V^T P^T : P stays in registers (the accumulator registers, converted, ARE the B
+//                 operand); V is staged untransposed [key][h] and read with the LDS transpose
+//                 loads, which deliver four consecutive keys of one h.  The row sum of P comes
+//                 from one more MFMA against a fragment of ones.
+// K and V tiles go from global memory straight into LDS (buffer_load ... lds), two stages,
+// the loads of block j+1 in flight while block j is computed.
+// Online softmax in the exp2 domain: the scale is folded into the exponent (one FMA per
+// element), the running reference max only moves when a block max exceeds it by more than
+// 2^8 (so O is rescaled in few blocks), and O is divided by l once at the end.  Causal: key >
+// query masked (top-left aligned), key blocks past the diagonal are never visited, work-groups
+// are issued heaviest first.
 #include <utility>
 
 #include "common.h"
@@ -28,10 +33,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
-constexpr int BR = 128;  // query rows per work-group
-constexpr int BC = 64;   // keys per step
-constexpr int NT = 256;
+constexpr int BC = 64;  // keys per step
 constexpr uint32_t kOob = 0x80000000u;
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -44,7 +48,9 @@ struct FmhaParams {
   float* lse;
   int H, F, T;
   int nqb;       // query blocks per unit
-  float scale2;  // head_scale * log2(e)
+  int total;     // work-groups with work: units * nqb
+  int per_xcd;   // ceil(total / 8)
+  float scale2;  // head_scale * log2(e), > 0
 };
 
 template <typename F, int... I>
@@ -62,16 +68,47 @@ template <> struct Elem<__bf16> {
   static __device__ __forceinline__ floatx16 mfma(vec8 a, vec8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // acc + a + b in fp32
+  static __device__ __forceinline__ float dot2_ones(__bf16 a, __bf16 b, float acc) {
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(v2{a, b}, v2{(__bf16)1.0f, (__bf16)1.0f}, acc, false);
+  }
 };
 template <> struct Elem<_Float16> {
   typedef f16x8 vec8;
   static __device__ __forceinline__ floatx16 mfma(vec8 a, vec8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ float dot2_ones(_Float16 a, _Float16 b, float acc) {
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(v2{a, b}, v2{(_Float16)1.0f, (_Float16)1.0f}, acc, false);
+  }
 };
 
 __device__ __forceinline__ floatx16 zero16() {
   return floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+}
+
+// x *= alpha for an MFMA accumulator that stays in the accumulator registers.  Written out so
+// that the register allocator keeps the accumulators in one register file through the rare
+// rescale path instead of moving all of them between files in every iteration.  The leading
+// and trailing waits cover the MFMA -> VALU and VALU -> MFMA hazards, which the compiler
+// cannot see through the asm text.
+__device__ __forceinline__ void scale_acc(floatx16& x, float alpha) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    float e = x[i], tmp;
+    if (i == 0)
+      asm volatile("s_nop 7\n s_nop 7\n s_nop 7\n s_nop 7\n v_accvgpr_read_b32 %1, %0\n v_mul_f32 %1, %1, %2\n v_accvgpr_write_b32 %0, %1"
+                   : "+a"(e), "=&v"(tmp) : "v"(alpha));
+    else if (i == 15)
+      asm volatile("v_accvgpr_read_b32 %1, %0\n v_mul_f32 %1, %1, %2\n v_accvgpr_write_b32 %0, %1\n s_nop 7\n s_nop 7"
+                   : "+a"(e), "=&v"(tmp) : "v"(alpha));
+    else
+      asm volatile("v_accvgpr_read_b32 %1, %0\n v_mul_f32 %1, %1, %2\n v_accvgpr_write_b32 %0, %1"
+                   : "+a"(e), "=&v"(tmp) : "v"(alpha));
+    x[i] = e;
+  }
 }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
@@ -80,25 +117,38 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 __device__ __forceinline__ u32x4 buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff) {
   return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
 }
+// s_waitcnt immediate (gfx9 encoding): vmcnt(n), lgkmcnt(0), expcnt untouched.
+__host__ __device__ constexpr int wait_vm_lgkm0(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4); }
 
-// T: element type; HP: head size padded to 64 / 128 / 256.
-template <typename T, int HP, bool CAUSAL, bool BIAS>
-__global__ __launch_bounds__(NT, (HP <= 128 ? 2 : 1)) void fmha_fwd_kernel(FmhaParams p) {
+// T: element type; HP: head size padded to 64 / 128 / 256; QT: 32-row query tiles per wave;
+// NW: waves per work-group; WPS: waves per SIMD the register budget is set for.
+template <typename T, int HP, int QT, int NW, int WPS, bool CAUSAL, bool BIAS>
+__global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   typedef typename Elem<T>::vec8 V8;
-  constexpr int KCH = HP / 8;              // 16-byte chunks per K/V row
-  constexpr int NCH = BC * KCH / NT;       // chunks per thread per tile
-  constexpr int K_ROW = HP * 2;            // K tile row, bytes (chunks XOR-swizzled by row)
-  constexpr int V_ROW = HP * 2 + 64;       // V tile row, bytes (padded)
-  constexpr int K_BYTES = BC * K_ROW, V_BYTES = BC * V_ROW;
-  constexpr int STAGE = K_BYTES + V_BYTES;
-  constexpr int KS = HP / 16;              // k-steps of the S product
-  constexpr int HT = HP / 32;              // 32-wide h tiles of O
-  __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
+  constexpr int BR = NW * QT * 32;           // query rows per work-group
+  constexpr int ROWB = HP * 2;               // bytes of one K / V row in LDS
+  constexpr int CPR = ROWB / 16;             // 16-byte chunks per row
+  constexpr int KMASK = CPR >= 16 ? 15 : 7;  // K rows: chunk ^= key & KMASK (16 lanes -> 16 bank groups)
+  constexpr int TILE = BC * ROWB;            // one K or V tile
+  constexpr int RPL = 1024 / ROWB;           // tile rows per 1 KiB load
+  constexpr int NL = TILE / 1024 / NW;       // loads per wave per tile
+  constexpr int LROWS = NW * RPL;            // tile rows between consecutive loads of a wave
+  constexpr int KV = (LROWS % (KMASK + 1) == 0) ? 1 : 2;  // distinct K swizzles among a wave's loads
+  constexpr int KS = HP / 16;                // k-steps of the S product
+  constexpr int HT = HP / 32;                // 32-wide h tiles of O
+  static_assert(NL >= 1 && LROWS % 8 == 0 && (2 * LROWS) % (KMASK + 1) == 0, "tile / wave split");
+  __shared__ __attribute__((aligned(1024))) char lds[4 * TILE];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5, l32 = lane & 31;
-  const int unit = blockIdx.x / p.nqb;
-  const int qb = p.nqb - 1 - blockIdx.x % p.nqb;  // heaviest (latest) query blocks first
+  // Work-groups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD a
+  // contiguous range of (unit, query block) pairs, so that the query blocks of one unit, which
+  // stream the same K and V, run on one XCD at about the same time.
+  const int wg = (int)(blockIdx.x % 8) * p.per_xcd + (int)(blockIdx.x / 8);
+  if (wg >= p.total) return;
+  const int unit = wg / p.nqb;
+  const int qb = p.nqb - 1 - wg % p.nqb;  // heaviest (latest) query blocks first
   const int q0 = qb * BR;
   const int H = p.H, F = p.F, Tk = p.T;
 
@@ -106,210 +156,311 @@ __global__ __launch_bounds__(NT, (HP <= 128 ? 2 : 1)) void fmha_fwd_kernel(FmhaP
   const T* K = reinterpret_cast<const T*>(p.k) + (int64_t)unit * Tk * H;
   const T* V = reinterpret_cast<const T*>(p.v) + (int64_t)unit * Tk * H;
 
-  // ---- Q fragments (B operand of S^T): lane holds query row `qrow`, h = 16 s + 8 g .. +7.
-  const int qrow = q0 + wave * 32 + l32;
-  V8 qf[KS];
+  // ---- Q fragments (B operand of S^T): tile t of this wave holds query rows wq0 + 32 t + l%32,
+  // fragment s covers h = 16 s + 8 g .. +7.
+  const int wq0 = q0 + wave * (QT * 32);
+  V8 qf[QT][KS];
   {
     const int rows_left = F - q0;  // > 0
     const __amdgpu_buffer_rsrc_t rq = make_rsrc(Q + (int64_t)q0 * H, (uint32_t)rows_left * H * 2);
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int h = 16 * s + 8 * g;
-      const uint32_t off = h < H ? (uint32_t)(((wave * 32 + l32) * H + h) * 2) : kOob;
-      qf[s] = __builtin_bit_cast(V8, buf_load(rq, off));
+    for (int t = 0; t < QT; ++t)
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int h = 16 * s + 8 * g;
+        const int r = wave * (QT * 32) + 32 * t + l32;
+        const uint32_t off = h < H ? (uint32_t)((r * H + h) * 2) : kOob;  // rows past F are out of range
+        qf[t][s] = __builtin_bit_cast(V8, buf_load(rq, off));
+      }
+  }
+
+  // ---- K / V tile loads, global -> LDS.  Load j = i * NW + wave fills LDS bytes [1024 j, +1024)
+  // of the tile, i.e. tile rows j * RPL ..; lane l lands at row j * RPL + l / CPR, chunk l % CPR,
+  // and fetches the global chunk that belongs there under the tile's swizzle.
+  const int lrow = wave * RPL + lane / CPR;  // tile row of this lane in load 0; load i: + i * LROWS
+  uint32_t koff[KV];
+#pragma unroll
+  for (int v = 0; v < KV; ++v) {
+    const int row = lrow + v * LROWS;
+    const int chunk = (lane % CPR) ^ (row & KMASK);
+    koff[v] = chunk * 8 < H ? (uint32_t)((lrow * H + chunk * 8) * 2) : kOob;
+  }
+  // V rows: chunk ^= vswz(key).  A transpose read touches 4 chunks of each of 4 consecutive keys;
+  // the XOR moves each key's group of 4 chunks to its own banks.
+  auto vswz = [](int key) { return CPR >= 16 ? (key & 3) << 2 : (key & 2) << 1; };
+  const int vchunk = (lane % CPR) ^ vswz(lrow);
+  const uint32_t voff = vchunk * 8 < H ? (uint32_t)((lrow * H + vchunk * 8) * 2) : kOob;
+  const uint32_t lstride = (uint32_t)(LROWS * H * 2);  // global bytes between a wave's loads
+  // One tile (64 rows from row t0 of K or V) into `tile`.  The per-load scalar offset is not
+  // range-checked by the hardware, so in the one ragged block rows past T are turned into
+  // out-of-range lane offsets, which load zeros.
+  auto issue_tile = [&](const T* base, int t0, char* __restrict__ tile, const uint32_t* offs, int noffs) {
+    const int rows_left = Tk - t0;  // > 0
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)t0 * H, 0x7fffffffu);
+    const bool full = rows_left >= BC;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const uint32_t off = (full || lrow + i * LROWS < rows_left) ? offs[i % noffs] : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(tile + (i * NW + wave) * 1024), 16, off,
+                                               i * lstride, 0, 0);
+    }
+  };
+
+  // ---- per-lane LDS offsets of the fragments
+  // K fragment (kt, s): key row 32 kt + l%32, logical chunk 2 s + g.
+  int kbase[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) kbase[s] = l32 * ROWB + (((2 * s + g) ^ (l32 & KMASK)) << 4);
+  // V^T fragment (group u, h tile ht): two transpose reads; within a 16-lane block lane pl
+  // addresses key row 16 u + 4 g + pl/4 (+8 for the second read), h = cb + 4 (pl%4) .. +3.
+  int vbase[HT][2];
+  {
+    const int pl = lane & 15;
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht) {
+      const int col = 32 * ht + ((lane >> 4) & 1) * 16 + 4 * (pl & 3);
+      const int chunk = col >> 3, within = (col & 7) * 2;
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const int key = 4 * g + (pl >> 2) + 8 * h2;  // + 16 u: does not change key & 3
+        vbase[ht][h2] = key * ROWB + ((chunk ^ vswz(key)) << 4) + within;
+      }
     }
   }
 
-  // ---- staging of K / V tiles: chunk ch = tid + i NT -> key row ch / KCH, chunk ch % KCH.
-  uint32_t voff[NCH];
-  int koff[NCH], vlds[NCH];
+  floatx16 ot[QT][HT];
+  float m_run[QT], l_run[QT];  // l_run: this lane's share (its 32 keys of every block) of the row sum
 #pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int ch = tid + i * NT;
-    const int row = ch / KCH, c = ch % KCH;
-    voff[i] = c * 8 < H ? (uint32_t)((row * H + c * 8) * 2) : kOob;
-    koff[i] = row * K_ROW + ((c ^ (row & 7)) << 4);
-    vlds[i] = row * V_ROW + (c << 4);
+  for (int t = 0; t < QT; ++t) {
+    m_run[t] = -INFINITY;
+    l_run[t] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < HT; ++i) ot[t][i] = zero16();
   }
-  u32x4 kr[NCH], vr[NCH];
-  auto load_tiles = [&](int t0) {
-    const uint32_t bytes = (uint32_t)(Tk - t0) * H * 2;  // rows past T read as zero
-    const __amdgpu_buffer_rsrc_t rk = make_rsrc(K + (int64_t)t0 * H, bytes);
-    const __amdgpu_buffer_rsrc_t rv = make_rsrc(V + (int64_t)t0 * H, bytes);
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) kr[i] = buf_load(rk, voff[i]);
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) vr[i] = buf_load(rv, voff[i]);
-  };
-  auto store_tiles = [&](char* stage) {
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) *reinterpret_cast<u32x4*>(stage + koff[i]) = kr[i];
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) *reinterpret_cast<u32x4*>(stage + K_BYTES + vlds[i]) = vr[i];
-  };
-
-  floatx16 ot[HT];
-#pragma unroll
-  for (int i = 0; i < HT; ++i) ot[i] = zero16();
-  float m_run = -INFINITY, l_run = 0.0f;
+  const float inv_scale = kLog2e / p.scale2;  // bias is added in score units: (s + b / scale) * scale
 
   const int kend = CAUSAL ? min(Tk, q0 + BR) : Tk;  // keys this work-group can see
   const int nblk = (kend + BC - 1) / BC;
-  const int wq_min = q0 + wave * 32, wq_max = wq_min + 31;
 
-  load_tiles(0);
-  store_tiles(lds);
-  __syncthreads();
-
-  for (int it = 0; it < nblk; ++it) {
-    const int t0 = it * BC;
-    const char* ks_ = lds + (it & 1) * STAGE;
-    const char* vs_ = ks_ + K_BYTES;
-    const bool more = it + 1 < nblk;
-    if (more) load_tiles(t0 + BC);
-
-    if (!CAUSAL || t0 <= wq_max) {  // wave-uniform: this wave has at least one visible key
-      // ---- S^T = K Q^T, two 32-key tiles
-      floatx16 st[2];
-      st[0] = zero16();
-      st[1] = zero16();
+  // S^T = K Q^T of one key block for all query tiles; each K fragment is read once.
+  auto scores = [&](const char* __restrict__ ktile, floatx16 (&st)[QT][2]) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
+    for (int t = 0; t < QT; ++t) { st[t][0] = zero16(); st[t][1] = zero16(); }
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-          const int row = kt * 32 + l32;
-          const int c = 2 * s + g;
-          const u32x4 kv =
-              *reinterpret_cast<const u32x4*>(ks_ + row * K_ROW + ((c ^ (row & 7)) << 4));
-          st[kt] = Elem<T>::mfma(__builtin_bit_cast(V8, kv), qf[s], st[kt]);
-        }
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const u32x4 kv = *reinterpret_cast<const u32x4*>(ktile + kbase[s] + kt * 32 * ROWB);
+#pragma unroll
+        for (int t = 0; t < QT; ++t) st[t][kt] = Elem<T>::mfma(__builtin_bit_cast(V8, kv), qf[t][s], st[t][kt]);
       }
-      // ---- scale (+ bias), masks.  st[kt][i] <-> key t0 + 32 kt + 8 (i/4) + 4 g + i%4.
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) st[kt][i] *= p.scale2;
-      if constexpr (BIAS) {
-        if (qrow < F) {
-          const T* bp = reinterpret_cast<const T*>(p.bias) + ((int64_t)unit * F + qrow) * Tk;
-#pragma unroll
-          for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int key = t0 + 32 * kt + 8 * (i / 4) + 4 * g + (i % 4);
-              if (key < Tk) st[kt][i] += kLog2e * (float)bp[key];
-            }
-        }
-      }
-      const bool diag = CAUSAL && (t0 + BC - 1 > wq_min);
-      const bool tail = t0 + BC > Tk;
-      if (diag || tail) {
+  };
+
+  // Bias, masks, block max and (rarely) the rescale of tile t; returns the exponent reference.
+  // st[kt][i] <-> key t0 + 32 kt + 8 (i/4) + 4 g + i%4.  Scores stay unscaled; the scale is
+  // folded into the exponent.
+  auto prepare = [&](auto TI, floatx16 (&st)[2], int t0) -> float {
+    constexpr int t = decltype(TI)::value;
+    const int qrow = wq0 + 32 * t + l32;
+    if constexpr (BIAS) {
+      if (qrow < F) {
+        const T* bp = reinterpret_cast<const T*>(p.bias) + ((int64_t)unit * F + qrow) * Tk;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const int key = t0 + 32 * kt + 8 * (i / 4) + 4 * g + (i % 4);
-            if ((CAUSAL && key > qrow) || key >= Tk) st[kt][i] = -INFINITY;
+            if (key < Tk) st[kt][i] += (float)bp[key] * inv_scale;
           }
       }
-      // ---- online softmax for this lane's query row
-      float mx = st[0][0];
-#pragma unroll
-      for (int i = 1; i < 16; ++i) mx = fmaxf(mx, st[0][i]);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, st[1][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // first block: exp2(-inf) = 0
-      float rs = 0.0f;
+    }
+    const bool diag = CAUSAL && (t0 + BC - 1 > wq0 + 32 * t);
+    const bool tail = t0 + BC > Tk;
+    if (diag || tail) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          st[kt][i] = __builtin_amdgcn_exp2f(st[kt][i] - m_new);
-          rs += st[kt][i];
+          const int key = t0 + 32 * kt + 8 * (i / 4) + 4 * g + (i % 4);
+          if ((CAUSAL && key > qrow) || key >= Tk) st[kt][i] = -INFINITY;
         }
-      l_run = l_run * alpha + rs;
-      m_run = m_new;
+    }
+    // The reference max m_run only moves when some row's block max exceeds it by more than 2^8
+    // (wave-uniform test): P then stays below 256, and O is rescaled in few blocks instead of all.
+    float mx = fmaxf(st[0][0], st[0][1]);
 #pragma unroll
-      for (int ht = 0; ht < HT; ++ht)
+    for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, st[0][i]), st[0][i + 1]);  // v_max3_f32
 #pragma unroll
-        for (int i = 0; i < 16; ++i) ot[ht][i] *= alpha;
-      // ---- O^T += V^T P^T.  MFMA (kt, hf) contracts keys 32 kt + 16 hf + {0..3, 8..11} + 4 g.
+    for (int i = 0; i < 16; i += 2) mx = fmaxf(fmaxf(mx, st[1][i]), st[1][i + 1]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float mx2 = mx * p.scale2;
+    if (__any(mx2 > m_run[t] + 8.0f)) {
+      const float m_new = fmaxf(m_run[t], mx2);
+      const float alpha = __builtin_amdgcn_exp2f(m_run[t] - m_new);  // first block: exp2(-inf) = 0
+      m_run[t] = m_new;
+      l_run[t] *= alpha;
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
+      for (int ht = 0; ht < HT; ++ht) scale_acc(ot[t][ht], alpha);
+    }
+    // A row that has seen no visible key keeps m_run = -inf; use 0 as its reference so that
+    // its masked (-inf) scores give exp2(-inf) = 0 and not NaN.
+    return m_run[t] == -INFINITY ? 0.0f : m_run[t];
+  };
+
+  // P = exp2(s * scale2 - mref) of one tile as four B-operand fragments (group u contracts keys
+  // 16 u + {0..3, 8..11} + 4 g), and the lane's row-sum share, summed from the rounded values
+  // the P V product uses.
+  auto probs = [&](const floatx16 (&st)[2], float mref, V8 (&pf)[4], float& lsum) {
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          V8 pf;
+    for (int u = 0; u < 4; ++u) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) pf[j] = (T)st[kt][8 * hf + j];
-          const int pl = lane & 15;
-          const int kb = 32 * kt + 16 * hf + 4 * g;
+      for (int j = 0; j < 8; ++j)
+        pf[u][j] = (T)__builtin_amdgcn_exp2f(__builtin_fmaf(st[u >> 1][8 * (u & 1) + j], p.scale2, -mref));
 #pragma unroll
-          for (int ht = 0; ht < HT; ++ht) {
-            const int cb = 32 * ht + ((lane >> 4) & 1) * 16;
-            const char* a0 = vs_ + (kb + (pl >> 2)) * V_ROW + (cb + 4 * (pl & 3)) * 2;
-            typedef short4v __attribute__((address_space(3))) * lds_ptr;
-            const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(a0));
-            const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(a0 + 8 * V_ROW));
-            u32x4 vv;
-            vv[0] = __builtin_bit_cast(u32x2, lo)[0];
-            vv[1] = __builtin_bit_cast(u32x2, lo)[1];
-            vv[2] = __builtin_bit_cast(u32x2, hi)[0];
-            vv[3] = __builtin_bit_cast(u32x2, hi)[1];
-            ot[ht] = Elem<T>::mfma(__builtin_bit_cast(V8, vv), pf, ot[ht]);
+      for (int j = 0; j < 8; j += 2) lsum = Elem<T>::dot2_ones(pf[u][j], pf[u][j + 1], lsum);
+    }
+  };
+
+  // O^T += V^T P^T for tile t.
+  auto accumulate = [&](auto TI, const char* __restrict__ vtile, const V8 (&pf)[4]) {
+    constexpr int t = decltype(TI)::value;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int ht = 0; ht < HT; ++ht) {
+        typedef short4v __attribute__((address_space(3))) * lds_ptr;
+        const char* vt = vtile + u * 16 * ROWB;
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + vbase[ht][0]));
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + vbase[ht][1]));
+        u32x4 vv;
+        vv[0] = __builtin_bit_cast(u32x2, lo)[0];
+        vv[1] = __builtin_bit_cast(u32x2, lo)[1];
+        vv[2] = __builtin_bit_cast(u32x2, hi)[0];
+        vv[3] = __builtin_bit_cast(u32x2, hi)[1];
+        ot[t][ht] = Elem<T>::mfma(__builtin_bit_cast(V8, vv), pf[u], ot[t][ht]);
+      }
+  };
+
+  // LDS: K tiles of blocks j, j+1 in kst[j & 1], V tiles in vst[j & 1].
+  char* const kst0 = lds;
+  char* const vst0 = lds + 2 * TILE;
+
+  // Prologue: K_0, then K_1 and V_0; S_0 is computed as soon as K_0 is there.
+  issue_tile(K, 0, kst0, koff, KV);
+  if (nblk > 1) issue_tile(K, BC, kst0 + TILE, koff, KV);
+  issue_tile(V, 0, vst0, &voff, 1);
+  if (nblk > 1) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(2 * NL));
+  else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(NL));
+  __builtin_amdgcn_s_barrier();
+  floatx16 st_a[QT][2], st_b[QT][2];
+  scores(kst0, st_a);
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  __builtin_amdgcn_s_barrier();
+
+  // One key block j: `sc` holds S_j; K_{j+1} and V_j are in LDS.  Loads of K_{j+2} and V_{j+1}
+  // are issued first and land during the block.  S_{j+1} (MFMA) is issued among the exponentials
+  // of tile 0 (VALU), the P V product of tile 0 among those of tile 1.  The four tile pointers
+  // never overlap (__restrict__), so the compiler does not make the fragment reads wait for the
+  // loads in flight.
+  auto block = [&](int it, floatx16 (&sc)[QT][2], floatx16 (&sn)[QT][2], const char* __restrict__ knext,
+                   const char* __restrict__ vcur, char* __restrict__ kfree, char* __restrict__ vfree) {
+    const int t0 = it * BC;
+    if (it + 2 < nblk) issue_tile(K, t0 + 2 * BC, kfree, koff, KV);
+    if (it + 1 < nblk) issue_tile(V, t0 + BC, vfree, &voff, 1);
+    float mref[QT];
+    static_for<QT>([&](auto TI) { mref[decltype(TI)::value] = prepare(TI, sc[decltype(TI)::value], t0); });
+    V8 pf[QT][4];
+    // Past the last block this reads a stale tile: finite or not, S_{nblk} is never used.
+    scores(knext, sn);
+    probs(sc[0], mref[0], pf[0], l_run[0]);
+    static_for<QT>([&](auto TI) {
+      constexpr int t = decltype(TI)::value;
+      accumulate(TI, vcur, pf[t]);
+      if constexpr (t + 1 < QT) probs(sc[t + 1], mref[t + 1], pf[t + 1], l_run[t + 1]);
+    });
+    if constexpr (QT == 1) {
+      // Issue order for the scheduler: LDS fragment reads run three MFMAs ahead of their use, the
+      // exponentials are spread under the S MFMAs, and the copies of S_{j+1} out of the
+      // accumulator registers under the P V MFMAs.
+      constexpr int NS = 2 * KS, NP = 4 * HT, AHEAD = 3;  // MFMAs of S and of P V
+      constexpr int VALU_S = (32 + 32 + 16 + 16 + NS - 1) / NS;
+      __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+      static_for<NS>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, i + AHEAD < NS ? 1 : 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, VALU_S, 0);
+      });
+      static_for<NP>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if constexpr (i + AHEAD < NP) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (32 + NP - 1) / NP, 0);
+      });
+    }
+    // K_{j+2} and V_{j+1} have landed (this wave's loads; every wave's after the barrier), and
+    // this wave is done reading the tiles the next block's loads overwrite.
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+    __builtin_amdgcn_s_barrier();
+  };
+
+  for (int it = 0; it < nblk; it += 2) {
+    // K_{it+1} sits in K stage 1, V_it in V stage 0; K_{it+2} goes to K stage 0, V_{it+1} to V stage 1.
+    block(it, st_a, st_b, kst0 + TILE, vst0, kst0, vst0 + TILE);
+    if (it + 1 < nblk) block(it + 1, st_b, st_a, kst0, vst0 + TILE, kst0 + TILE, vst0);
+  }
+
+  // ---- finish: O = O^T / l; LSE = m ln2 + ln l.
+  static_for<QT>([&](auto TI) {
+    constexpr int t = decltype(TI)::value;
+    const int qrow = wq0 + 32 * t + l32;
+    const float l_tot = l_run[t] + __shfl_xor(l_run[t], 32);
+    const float inv = 1.0f / l_tot;
+    if (qrow < F) {
+      T* orow = reinterpret_cast<T*>(p.out) + ((int64_t)unit * F + qrow) * H;
+      static_for<HT>([&](auto HTI) {
+        constexpr int ht = decltype(HTI)::value;
+        const floatx16 o = ot[t][ht];
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const int h = 32 * ht + 8 * qd + 4 * g;
+          if (h < H) {  // H % 8 == 0, so the four values are all in range
+            union { T e[4]; u32x2 w; } r;
+            r.e[0] = (T)(o[4 * qd + 0] * inv);
+            r.e[1] = (T)(o[4 * qd + 1] * inv);
+            r.e[2] = (T)(o[4 * qd + 2] * inv);
+            r.e[3] = (T)(o[4 * qd + 3] * inv);
+            *reinterpret_cast<u32x2*>(orow + h) = r.w;
           }
         }
-      }
+      });
+      if (p.lse && g == 0) p.lse[(int64_t)unit * F + qrow] = m_run[t] * 0.6931471805599453f + logf(l_tot);
     }
-
-    if (more) store_tiles(lds + ((it + 1) & 1) * STAGE);
-    __syncthreads();
-  }
-
-  // ---- finish: l = both halves' partial sums; O = O^T / l; LSE = m ln2 + ln l.
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
-  const float inv = 1.0f / l_tot;
-  if (qrow < F) {
-    T* orow = reinterpret_cast<T*>(p.out) + ((int64_t)unit * F + qrow) * H;
-    static_for<HT>([&](auto HTI) {
-      constexpr int ht = decltype(HTI)::value;
-      const floatx16 t = ot[ht];
-#pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int h = 32 * ht + 8 * qd + 4 * g;
-        if (h < H) {  // H % 8 == 0, so the four values are all in range
-          union { T e[4]; u32x2 w; } o;
-          o.e[0] = (T)(t[4 * qd + 0] * inv);
-          o.e[1] = (T)(t[4 * qd + 1] * inv);
-          o.e[2] = (T)(t[4 * qd + 2] * inv);
-          o.e[3] = (T)(t[4 * qd + 3] * inv);
-          *reinterpret_cast<u32x2*>(orow + h) = o.w;
-        }
-      }
-    });
-    if (p.lse && g == 0) p.lse[(int64_t)unit * F + qrow] = m_run * 0.6931471805599453f + logf(l_tot);
-  }
+  });
 }
 
-template <typename T, int HP>
-void launch_hp(const FmhaParams& p, int units, bool causal, bool bias, hipStream_t st) {
-  const dim3 grid((unsigned)(units * p.nqb)), block(NT);
+template <typename T, int HP, int QT, int NW, int WPS>
+void launch_cfg(FmhaParams p, uint64_t units, uint32_t F, bool causal, bool bias, hipStream_t st) {
+  p.nqb = (int)((F + NW * QT * 32 - 1) / (NW * QT * 32));
+  p.total = (int)(units * p.nqb);
+  p.per_xcd = (p.total + 7) / 8;
+  const dim3 grid((unsigned)(p.per_xcd * 8)), block(NW * 64);
   if (causal) {
-    if (bias) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, true, true>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, true, false>), grid, block, 0, st, p);
+    if (bias) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, true, true>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, true, false>), grid, block, 0, st, p);
   } else {
-    if (bias) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, false, true>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, false, false>), grid, block, 0, st, p);
+    if (bias) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, false, true>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, false, false>), grid, block, 0, st, p);
   }
 }
 
 template <typename T>
-void launch_t(const FmhaParams& p, int units, bool causal, bool bias, hipStream_t st) {
-  // Head-size classes of the reference's policy choice (fmha_forward.h:622-646).
-  if (p.H <= 64) launch_hp<T, 64>(p, units, causal, bias, st);
-  else if (p.H <= 128) launch_hp<T, 128>(p, units, causal, bias, st);
-  else launch_hp<T, 256>(p, units, causal, bias, st);
+void launch_t(const FmhaParams& p, uint64_t units, uint32_t F, bool causal, bool bias, hipStream_t st) {
+  // Head-size classes of the reference's policy choice (fmha_forward.h:622-646).  Two query tiles
+  // per wave where the accumulators fit in the register file (head size <= 128).
+  if (p.H <= 64) launch_cfg<T, 64, 1, 4, 2>(p, units, F, causal, bias, st);
+  else if (p.H <= 128) launch_cfg<T, 128, 1, 4, 2>(p, units, F, causal, bias, st);
+  else launch_cfg<T, 256, 1, 4, 1>(p, units, F, causal, bias, st);
 }
 
 }  // namespace
@@ -327,9 +478,10 @@ extern "C" int xmk_fmha_fwd(const void* query, const void* key, const void* valu
     return xmk::fail(XMK_UNIMPLEMENTED, "fmha_fwd: head_size %u > 256 (fmha_forward.h:642)", head_size);
   if (head_size % 8 != 0)
     return xmk::fail(XMK_UNIMPLEMENTED, "fmha_fwd: head_size %u is not a multiple of 8", head_size);
+  if (!(head_scale > 0.0f) || head_scale > 3.0e38f)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_fwd: head_scale must be positive and finite");
   const uint64_t units = (uint64_t)num_batches * num_heads;
-  const uint64_t nqb = (num_queries + BR - 1) / BR;
-  if (units * nqb > 0x7fffffffull || (uint64_t)num_keys * head_size * 2 >= kOob ||
+  if (units * ((num_queries + 31) / 32) > 0x7fffffffull || (uint64_t)num_keys * head_size * 2 >= kOob ||
       (uint64_t)num_queries * head_size * 2 >= kOob)
     return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_fwd: shape too large");
   if (!xmk::aligned(query, 16) || !xmk::aligned(key, 16) || !xmk::aligned(value, 16) ||
@@ -338,12 +490,12 @@ extern "C" int xmk_fmha_fwd(const void* query, const void* key, const void* valu
   FmhaParams p;
   p.q = query; p.k = key; p.v = value; p.bias = bias; p.out = out; p.lse = lse;
   p.H = (int)head_size; p.F = (int)num_queries; p.T = (int)num_keys;
-  p.nqb = (int)nqb;
+  p.nqb = p.total = p.per_xcd = 0;
   p.scale2 = head_scale * kLog2e;
   xmk::trace("fmha_fwd B=%u N=%u F=%u T=%u H=%u causal=%d bias=%d lse=%d", num_batches, num_heads,
              num_queries, num_keys, head_size, causal, bias != nullptr, lse != nullptr);
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == XMK_BF16) launch_t<__bf16>(p, (int)units, causal != 0, bias != nullptr, st);
-  else launch_t<_Float16>(p, (int)units, causal != 0, bias != nullptr, st);
+  if (dtype == XMK_BF16) launch_t<__bf16>(p, units, num_queries, causal != 0, bias != nullptr, st);
+  else launch_t<_Float16>(p, units, num_queries, causal != 0, bias != nullptr, st);
   return xmk::check_launch("fmha_fwd");
 }
