@@ -1,0 +1,61 @@
+"""The C-ABI library loads without a GPU and exports every entry point declared in include/xmk.h.
+
+No compute entry point is called here; argument validation that returns before any device work
+(null descriptors, bad dtypes) is exercised because it must hold on a host without a GPU too."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "xmk.h")
+LIB = os.path.join(ROOT, "intel-extension-for-openxla_amd", "libxmk.so")
+
+
+def declared_entry_points():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    # function declarations at file scope: "<type> xmk_name(" not preceded by typedef
+    names = re.findall(r"^\s*(?:const\s+)?[A-Za-z_][A-Za-z0-9_]*\s*\*?\s*(xmk_[a-z0-9_]+)\s*\(", text, flags=re.M)
+    return sorted(set(names))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        pytest.fail(f"{LIB} is not built; run __graft_entry__.build()")
+    return ctypes.CDLL(LIB)
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_entry_points()
+    for required in ("xmk_gemm", "xmk_fmha_fwd", "xmk_int4_gemm", "xmk_int4_dequant", "xmk_fp8_gemm",
+                     "xmk_fmha_decode", "xmk_gptj_decode_step", "xmk_last_error", "xmk_version"):
+        assert required in names, names
+
+
+def test_every_declared_symbol_is_exported(lib):
+    missing = [n for n in declared_entry_points() if not hasattr(lib, n)]
+    assert not missing, f"declared in xmk.h but not exported: {missing}"
+
+
+def test_version_and_error_strings(lib):
+    lib.xmk_version.restype = ctypes.c_char_p
+    lib.xmk_last_error.restype = ctypes.c_char_p
+    assert lib.xmk_version().decode().strip() != ""
+    assert isinstance(lib.xmk_last_error().decode(), str)
+
+
+def test_null_arguments_are_rejected_before_any_device_work(lib):
+    lib.xmk_last_error.restype = ctypes.c_char_p
+    lib.xmk_gemm.restype = ctypes.c_int
+    rc = lib.xmk_gemm(None, None)
+    assert rc == 3  # XMK_INVALID_ARGUMENT
+    assert lib.xmk_last_error().decode() != ""
+    lib.xmk_fmha_fwd.restype = ctypes.c_int
+    rc = lib.xmk_fmha_fwd(None, None, None, None, None, None, ctypes.c_int32(16), ctypes.c_uint32(1),
+                          ctypes.c_uint32(1), ctypes.c_uint32(64), ctypes.c_uint32(1), ctypes.c_uint32(1),
+                          ctypes.c_float(1.0), ctypes.c_int32(0), None)
+    assert rc == 3
