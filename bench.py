@@ -20,6 +20,17 @@ sys.path.insert(0, ROOT)
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0}  # dense MFMA TFLOP/s, MI355X
 HBM_PEAK = 8000.0                                        # GB/s
 
+# HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE (KiB per dispatch), FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0: the factors a
+# 1 GiB device copy (--workload copy) gives on this machine.  The runs are summarised in
+# profiles/hbm_traffic_pmc.txt; a workload without a measurement reports null.
+TRAFFIC_BYTES = {
+    "fmha_causal": (196700 * 2.0 + 131200) * 1024,
+    "gemm_8192": (790100 * 2.0 + 132800) * 1024,
+    "int4_m1": (17470 * 2.0 + 32) * 1024,
+    "fp8_8192": (416500 * 2.0 + 376000) * 1024,
+}
+
 
 def _events(torch, fn, steps, warmup, graph=False):
     """Average duration (ms) of fn over `steps` launches, HIP events on torch's current stream
@@ -147,7 +158,16 @@ def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
                 graph=True, graph_steps=3)
 
 
+def wl_copy(torch, xmk, nbytes=1 << 30):
+    """A plain device copy of known size: the calibration point for the HBM byte counters."""
+    src = torch.empty((nbytes,), dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    return dict(name=f"copy_{nbytes >> 20}MiB", fn=lambda: dst.copy_(src), flops=0.0, bytes=2.0 * nbytes,
+                bound="hbm", dtype="u8", kernel="torch copy kernel")
+
+
 WORKLOADS = {
+    "copy": lambda t, x: wl_copy(t, x),
     "fmha_causal": lambda t, x: wl_fmha(t, x, True),
     "fmha": lambda t, x: wl_fmha(t, x, False),
     "gemm_8192": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192),
@@ -172,7 +192,7 @@ def measure(torch, xmk, key, steps, warmup):
     else:
         achieved, peak, unit = w["bytes"] / ms / 1e6, HBM_PEAK, "GB/s"
     roof = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": None, "kernel": w["kernel"],
+            "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(key), "kernel": w["kernel"],
             "kernel_ms": round(ms, 5), "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]}
     return w, ms, wall_ms, roof
 
