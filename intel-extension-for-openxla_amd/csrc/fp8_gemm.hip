@@ -2,24 +2,28 @@
 //
 // MFMA kernel: A [M,K] row-major and B stored [N,K] (both reduction-contiguous, the
 // layout XLA's "__cublas$lt$matmul$f8" rewrite produces).  256x256 output tile per
-// work-group, K walked in steps of 128 bytes, operand tiles staged global -> registers
-// -> LDS (double-buffered, 16-byte chunks XOR-swizzled by row) and consumed by
-// v_mfma_f32_32x32x64_f8f6f4: a lane supplies 32 consecutive k of one row per
-// instruction.  The per-tensor scales are read from device memory in the epilogue.
+// work-group (2x2 waves), K walked in steps of 64 bytes = one v_mfma_f32_32x32x64_f8f6f4
+// k-step, in which a lane supplies 32 consecutive k of one row.  Operand tiles go from
+// global memory straight into LDS (buffer_load ... lds) through the same 4-stage ring,
+// swizzle and wait/barrier scheme as the 16-bit GEMM: a 64-byte fp8 row is byte for byte
+// the 32-element 16-bit row that kernel's loader handles.  The per-tensor scales are read
+// from device memory in the epilogue.
 // B stored [K,N] (rhs_transpose == 0) runs a plain tiled kernel.
 #include <utility>
 
-#include "common.h"
+#include "gemm_kernel.h"
 
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+using gemm_impl::floatx16;
+using gemm_impl::static_for;
+using gemm_impl::u32x2;
+using gemm_impl::u32x4;
+using gemm_impl::zero16;
 typedef int intx8 __attribute__((ext_vector_type(8)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int BKB = 128;  // K step in bytes (= fp8 elements)
-constexpr uint32_t kOob = 0x80000000u;
+constexpr int BKB = 64;  // K step in bytes (= fp8 elements)
+constexpr uint32_t kOob = gemm_impl::kOob;
 
 struct Fp8Params {
   const uint8_t* a;
@@ -31,82 +35,48 @@ struct Fp8Params {
   int tiles_m, tiles_n;
 };
 
-template <typename F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
-}
-
-__device__ __forceinline__ floatx16 zero16() {
-  return floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-}
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)kOob, 0x00020000);
-}
-
-// One operand tile [ROWS][128 bytes]: chunk ch = tid + i NT -> row ch / 8, 16-byte chunk ch % 8.
-template <int ROWS, int NT>
-struct Stager {
-  static constexpr int NCH = ROWS * 8 / NT;
-  u32x4 r[NCH];
-  uint32_t voff[NCH];
-  int kin;  // first k byte of this thread's chunks within the step (same for all chunks)
-
-  __device__ __forceinline__ void init(int64_t ld, int valid, int tid) {
-    kin = (tid % 8) * 16;
+// Per-lane LDS byte offsets of an operand's fragments: lane l of the 32-row slab t gets row
+// 32 t + l%32, bytes 32 (l/32) .. +31 of the 64-byte row, i.e. the two 16-byte chunks 2 (l/32)
+// and 2 (l/32) + 1, each XOR-swizzled like the loader placed them.  Adding 32 t rows does not
+// change the swizzle.
+struct Fp8Frag {
+  int base[2];
+  __device__ __forceinline__ void init(int row0, int lane) {
+    const int row = row0 + (lane & 31);
+    const int s = gemm_impl::swz<false, 0, 32>(row);
 #pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int row = (tid + i * NT) / 8;
-      voff[i] = row < valid ? (uint32_t)((int64_t)row * ld + kin) : kOob;
-    }
+    for (int h = 0; h < 2; ++h) base[h] = row * BKB + ((((lane >> 5) * 2 + h) ^ s) << 4);
   }
-  __device__ __forceinline__ void load(const void* base, int kleft) {
-    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base);
-    const bool ok = kin < kleft;  // K % 16 == 0: a chunk is all in or all out
-#pragma unroll
-    for (int i = 0; i < NCH; ++i)
-      r[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? voff[i] : kOob, 0, 0));
-  }
-  __device__ __forceinline__ void store(char* lds, int tid) const {
-#pragma unroll
-    for (int i = 0; i < NCH; ++i) {
-      const int ch = tid + i * NT;
-      const int row = ch / 8, c = ch % 8;
-      *reinterpret_cast<u32x4*>(lds + row * BKB + ((c ^ (row & 7)) << 4)) = r[i];
-    }
+  __device__ __forceinline__ intx8 read(const char* __restrict__ tile, int t) const {
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(tile + base[0] + t * 32 * BKB);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(tile + base[1] + t * 32 * BKB);
+    intx8 v;
+    v[0] = (int)lo[0]; v[1] = (int)lo[1]; v[2] = (int)lo[2]; v[3] = (int)lo[3];
+    v[4] = (int)hi[0]; v[5] = (int)hi[1]; v[6] = (int)hi[2]; v[7] = (int)hi[3];
+    return v;
   }
 };
-
-// Fragment for k-step ks (64 k): lane l gets row row0 + l%32, bytes 64 ks + 32 (l/32) .. +31.
-__device__ __forceinline__ intx8 read_frag(const char* lds, int row0, int ks, int lane) {
-  const int row = row0 + (lane & 31);
-  const int c = ks * 4 + (lane >> 5) * 2;
-  const u32x4 lo = *reinterpret_cast<const u32x4*>(lds + row * BKB + ((c ^ (row & 7)) << 4));
-  const u32x4 hi = *reinterpret_cast<const u32x4*>(lds + row * BKB + (((c + 1) ^ (row & 7)) << 4));
-  intx8 v;
-  v[0] = (int)lo[0]; v[1] = (int)lo[1]; v[2] = (int)lo[2]; v[3] = (int)lo[3];
-  v[4] = (int)hi[0]; v[5] = (int)hi[1]; v[6] = (int)hi[2]; v[7] = (int)hi[3];
-  return v;
-}
 
 __device__ __forceinline__ floatx16 mfma_fp8(intx8 a, intx8 b, floatx16 c) {
   // cbsz = blgp = 0: both operands e4m3; block scales 127 = 2^0 (E8M0).
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, 127);
 }
 
-template <int BM, int BN, int WGM, int WGN>
+template <int BM, int BN, int WGM, int WGN, int NSTAGE>
 __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
-  constexpr int NT = WGM * WGN * 64;
+  constexpr int NWAVES = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB, STAGE = A_BYTES + B_BYTES;
-  __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
+  // The loader works in 2-byte units: BK = 32 units = 64 bytes.
+  typedef gemm_impl::Loader<false, BM, 32, NWAVES> LoaderA;
+  typedef gemm_impl::Loader<false, BN, 32, NWAVES> LoaderB;
+  constexpr int LOADS = LoaderA::NL + LoaderB::NL;  // per wave per K step
+  static_assert(NSTAGE >= 3, "the barrier leaves the running step's loads in flight");
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
 
   int pid = blockIdx.x;
@@ -126,66 +96,84 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = zero16();
 
-  Stager<BM, NT> sa;
-  Stager<BN, NT> sb;
-  sa.init(p.K, p.M - m0, tid);
-  sb.init(p.K, p.N - n0, tid);
+  LoaderA la;
+  LoaderB lb;
+  la.init(p.K / 2, p.M - m0, wave, lane);
+  lb.init(p.K / 2, p.N - n0, wave, lane);
   const uint8_t* a_tile = p.a + (int64_t)m0 * p.K;
   const uint8_t* b_tile = p.b + (int64_t)n0 * p.K;
   const int KT = (p.K + BKB - 1) / BKB;
 
-  sa.load(a_tile, p.K);
-  sb.load(b_tile, p.K);
-  sa.store(lds, tid);
-  sb.store(lds + A_BYTES, tid);
-  __syncthreads();
-
-  intx8 fa[2][TM], fb[2][TN];
-  auto read_frags = [&](const char* stage, int ks, int buf) {
+  // Prologue: K steps 0 .. NSTAGE-2.  Loads past the end of K write zeros, so every step issues
+  // the same number of loads and the vmcnt arithmetic is uniform.
 #pragma unroll
-    for (int i = 0; i < TM; ++i) fa[buf][i] = read_frag(stage, wm * WTM + i * 32, ks, lane);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb[buf][j] = read_frag(stage + A_BYTES, wn * WTN + j * 32, ks, lane);
-  };
-  auto mma = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = mfma_fp8(fb[buf][j], fa[buf][i], acc[i][j]);
-  };
-  auto interleave = [&]() {
-#pragma unroll
-    for (int r = 0; r < 2 * (TM + TN); ++r) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-  };
-
-  read_frags(lds, 0, 0);
-  for (int kt = 0; kt < KT; ++kt) {
-    const char* cur = lds + (kt & 1) * STAGE;
-    char* nxt = lds + ((kt + 1) & 1) * STAGE;
-    const bool more = kt + 1 < KT;
-    if (more) {
-      a_tile += BKB;
-      b_tile += BKB;
-      sa.load(a_tile, p.K - (kt + 1) * BKB);
-      sb.load(b_tile, p.K - (kt + 1) * BKB);
-    }
-    read_frags(cur, 1, 1);
-    mma(0);
-    interleave();
-    __builtin_amdgcn_sched_barrier(0);
-    if (more) {
-      sa.store(nxt, tid);
-      sb.store(nxt + A_BYTES, tid);
-    }
-    __syncthreads();
-    if (more) read_frags(nxt, 0, 0);
-    mma(1);
-    if (more) interleave();
-    __builtin_amdgcn_sched_barrier(0);
+  for (int st = 0; st < NSTAGE - 1; ++st) {
+    la.issue(a_tile, (p.K - st * BKB) / 2, lds + st * STAGE, wave);
+    lb.issue(b_tile, (p.K - st * BKB) / 2, lds + st * STAGE + A_BYTES, wave);
+    a_tile += BKB;
+    b_tile += BKB;
   }
+  __builtin_amdgcn_s_waitcnt(gemm_impl::vmcnt_imm((NSTAGE - 2) * LOADS));  // step 0 has landed
+  __builtin_amdgcn_s_barrier();
+
+  Fp8Frag fa_addr, fb_addr;
+  fa_addr.init(wm * WTM, lane);
+  fb_addr.init(wn * WTN, lane);
+  // Fragment registers: the B fragments of a step are double-buffered (those of step kt + 1 are
+  // read while step kt computes); the A fragments rotate through two slots, A fragment i + 1
+  // being read under the MFMAs of fragment i, and fragment 0 of the next step under the last.
+  static_assert(TM % 2 == 0 && TN <= TM, "fragment rotation");
+  intx8 fa[2], fb[2][TN];
+  constexpr int NMFMA = TM * TN;
+  // One K step kt: B fragments (buffer `par`) and A fragment 0 of step kt are in registers.  Once
+  // step kt + 1 has landed for every wave (vmcnt + barrier; all reads issued so far are complete
+  // too), issue the loads of step kt + NSTAGE - 1 into the stage step kt - 1 used, and run the
+  // MFMAs of step kt while reading the rest of its A fragments from `cur` and the first fragments
+  // of step kt + 1 from `nxt`.  The stages are distinct (__restrict__), so the compiler keeps the
+  // loads in flight across the fragment reads.
+  auto k_step = [&](auto PAR, const char* __restrict__ cur, const char* __restrict__ nxt, char* __restrict__ wr,
+                    int kt) {
+    constexpr int par = decltype(PAR)::value;
+    const int kleft = (p.K - (kt + NSTAGE - 1) * BKB) / 2;
+    const __amdgpu_buffer_rsrc_t ra = gemm_impl::make_rsrc(a_tile), rb = gemm_impl::make_rsrc(b_tile);
+    __builtin_amdgcn_s_waitcnt(gemm_impl::vmcnt_imm((NSTAGE - 3) * LOADS) & ~(0xf << 8));  // and lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < LoaderA::NL; ++i) la.issue_one(i, ra, kleft, wr, wave);
+#pragma unroll
+    for (int i = 0; i < LoaderB::NL; ++i) lb.issue_one(i, rb, kleft, wr + A_BYTES, wave);
+    static_for<TM>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      if constexpr (i + 1 < TM) fa[(i + 1) & 1] = fa_addr.read(cur, i + 1);
+      else fa[0] = fa_addr.read(nxt, 0);
+      if constexpr (i < TN) fb[par ^ 1][i] = fb_addr.read(nxt + A_BYTES, i);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = mfma_fp8(fb[par][j], fa[i & 1], acc[i][j]);
+    });
+    // Issue order: each row of MFMAs starts with its LDS reads (4 x 16 bytes), the global loads
+    // are spread evenly.
+    static_for<NMFMA>([&](auto R) {
+      constexpr int r = decltype(R)::value;
+      if constexpr (r % TN == 0) __builtin_amdgcn_sched_group_barrier(0x100, (r / TN < TN) ? 4 : 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if constexpr ((r + 1) * LOADS / NMFMA > r * LOADS / NMFMA) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    a_tile += BKB;
+    b_tile += BKB;
+  };
+
+#pragma unroll
+  for (int j = 0; j < TN; ++j) fb[0][j] = fb_addr.read(lds + A_BYTES, j);
+  fa[0] = fa_addr.read(lds, 0);
+  for (int kt = 0; kt < KT; kt += 2) {
+    k_step(std::integral_constant<int, 0>{}, lds + (kt % NSTAGE) * STAGE, lds + ((kt + 1) % NSTAGE) * STAGE,
+           lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE, kt);
+    if (kt + 1 < KT)
+      k_step(std::integral_constant<int, 1>{}, lds + ((kt + 1) % NSTAGE) * STAGE,
+             lds + ((kt + 2) % NSTAGE) * STAGE, lds + ((kt + NSTAGE) % NSTAGE) * STAGE, kt + 1);
+  }
+  __builtin_amdgcn_s_waitcnt(gemm_impl::vmcnt_imm(0));  // drain the zero-fill loads before LDS is released
 
   // acc[i][j][e] is out[m][n], m = m0 + wm WTM + 32 i + lane%32, n = n0 + wn WTN + 32 j + 8 (e/4) + 4 (lane/32) + e%4.
   const float scale = p.a_scale[0] * p.b_scale[0];
@@ -276,10 +264,10 @@ extern "C" int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, 
                big ? "mfma_256x256" : "mfma_128x128");
     if (big) {
       p.tiles_m = (int)xmk::ceil_div(m, 256); p.tiles_n = (int)xmk::ceil_div(n, 256);
-      hipLaunchKernelGGL((fp8_gemm_kernel<256, 256, 2, 2>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
+      hipLaunchKernelGGL((fp8_gemm_kernel<256, 256, 2, 4, 4>), dim3(p.tiles_m * p.tiles_n), dim3(512), 0, st, p);
     } else {
       p.tiles_m = (int)xmk::ceil_div(m, 128); p.tiles_n = (int)xmk::ceil_div(n, 128);
-      hipLaunchKernelGGL((fp8_gemm_kernel<128, 128, 2, 2>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
+      hipLaunchKernelGGL((fp8_gemm_kernel<128, 128, 2, 2, 4>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
     }
   } else {
     xmk::trace("fp8_gemm m=%lld n=%lld k=%lld rhs_t=%d -> generic_64x64", (long long)m, (long long)n,

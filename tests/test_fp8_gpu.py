@@ -17,6 +17,7 @@ def _quant(oracle, shape, seed):
 
 @pytest.mark.parametrize("m,n,k,rhs_t", [
     (256, 256, 128, True), (512, 384, 1024, True), (300, 260, 208, True), (64, 8, 16, True),
+    (4136, 4104, 208, True),  # ragged edges of the 256x256 tile (taken when there are >= 256 tiles)
     (130, 72, 80, False), (256, 256, 256, False),
 ])
 def test_fp8_gemm_shapes(xmk, oracle, m, n, k, rhs_t):
