@@ -1,4 +1,5 @@
-"""The C-ABI library loads without a GPU and exports every entry point declared in include/xmk.h.
+"""The C-ABI library loads without a GPU and exports every entry point declared in include/xmk.h
+and include/xmk_ffi.h.
 
 No compute entry point is called here; argument validation that returns before any device work
 (null descriptors, bad dtypes) is exercised because it must hold on a host without a GPU too."""
@@ -9,12 +10,12 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "xmk.h")
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("xmk.h", "xmk_ffi.h")]
 LIB = os.path.join(ROOT, "intel-extension-for-openxla_amd", "libxmk.so")
 
 
 def declared_entry_points():
-    text = open(HEADER).read()
+    text = "\n".join(open(h).read() for h in HEADERS)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     text = re.sub(r"//[^\n]*", "", text)
     # function declarations at file scope: "<type> xmk_name(" not preceded by typedef
@@ -32,7 +33,10 @@ def lib():
 def test_header_declares_the_expected_surface():
     names = declared_entry_points()
     for required in ("xmk_gemm", "xmk_fmha_fwd", "xmk_int4_gemm", "xmk_int4_dequant", "xmk_fp8_gemm",
-                     "xmk_fmha_decode", "xmk_gptj_decode_step", "xmk_last_error", "xmk_version"):
+                     "xmk_fmha_decode", "xmk_gptj_decode_step", "xmk_last_error", "xmk_version",
+                     "xmk_ffi_cublas_gemm", "xmk_ffi_cublas_lt_matmul", "xmk_ffi_fmha_softmax",
+                     "xmk_ffi_fmha_scale_bias_softmax", "xmk_ffi_int4_gemm", "xmk_ffi_cublas_lt_matmul_f8",
+                     "xmk_ffi_targets", "xmk_ffi_register_all"):
         assert required in names, names
 
 
