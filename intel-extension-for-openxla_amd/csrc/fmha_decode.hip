@@ -153,26 +153,63 @@ __global__ __launch_bounds__(NT) void fmha_decode_split_kernel(DecodeParams p) {
   if (tid == 0) { wsu[H] = s_stat[0]; wsu[H + 1] = s_stat[1]; }
 }
 
+constexpr int MAXSPLITS = 1024;
+
+// Block-wide max / sum of one float per thread (NT threads); every thread gets the result.
+template <bool IS_MAX>
+__device__ __forceinline__ float block_reduce(float v, float* s_tmp) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    const float w = __shfl_xor(v, o);
+    v = IS_MAX ? fmaxf(v, w) : v + w;
+  }
+  __syncthreads();  // s_tmp may still be read from an earlier call
+  if ((threadIdx.x & 63) == 0) s_tmp[threadIdx.x >> 6] = v;
+  __syncthreads();
+  v = s_tmp[0];
+#pragma unroll
+  for (int i = 1; i < NT / 64; ++i) v = IS_MAX ? fmaxf(v, s_tmp[i]) : v + s_tmp[i];
+  return v;
+}
+
+// One work-group per unit: the weights 2^(m_s - m) / l of the splits are formed once in LDS
+// (thread s handles split s), then thread h adds up column h of the partial outputs with
+// independent, coalesced loads.
 template <typename T>
 __global__ __launch_bounds__(NT) void fmha_decode_merge_kernel(DecodeParams p) {
-  const int unit = blockIdx.x, H = p.H;
-  const float* wsu = p.ws + (int64_t)unit * p.splits * (H + 2);
+  __shared__ float s_w[MAXSPLITS];
+  __shared__ float s_tmp[NT / 64];
+  const int unit = blockIdx.x, H = p.H, S = p.splits;
+  const int64_t stride = H + 2;
+  const float* wsu = p.ws + (int64_t)unit * S * stride;
   float m = -INFINITY;
-  for (int s = 0; s < p.splits; ++s) m = fmaxf(m, wsu[(int64_t)s * (H + 2) + H]);
-  float l = 0.f;
-  for (int s = 0; s < p.splits; ++s) {
-    const float ms = wsu[(int64_t)s * (H + 2) + H];
-    if (ms > -INFINITY) l += wsu[(int64_t)s * (H + 2) + H + 1] * __builtin_amdgcn_exp2f(ms - m);
+  for (int s = threadIdx.x; s < S; s += NT) {
+    const float ms = wsu[s * stride + H];
+    s_w[s] = ms;
+    m = fmaxf(m, ms);
   }
+  m = block_reduce<true>(m, s_tmp);
+  float l = 0.f;
+  for (int s = threadIdx.x; s < S; s += NT) {
+    const float ms = s_w[s];  // written by this thread
+    const float w = ms > -INFINITY ? __builtin_amdgcn_exp2f(ms - m) : 0.f;
+    l += wsu[s * stride + H + 1] * w;
+    s_w[s] = w;
+  }
+  l = block_reduce<false>(l, s_tmp);  // its barriers also publish s_w
   const float inv = 1.0f / l;
   T* out = reinterpret_cast<T*>(p.out) + (int64_t)unit * H;
   for (int h = threadIdx.x; h < H; h += NT) {
-    float o = 0.f;
-    for (int s = 0; s < p.splits; ++s) {
-      const float ms = wsu[(int64_t)s * (H + 2) + H];
-      if (ms > -INFINITY) o += wsu[(int64_t)s * (H + 2) + h] * __builtin_amdgcn_exp2f(ms - m);
+    float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+    int s = 0;
+    for (; s + 4 <= S; s += 4) {
+      o0 += wsu[(s + 0) * stride + h] * s_w[s + 0];
+      o1 += wsu[(s + 1) * stride + h] * s_w[s + 1];
+      o2 += wsu[(s + 2) * stride + h] * s_w[s + 2];
+      o3 += wsu[(s + 3) * stride + h] * s_w[s + 3];
     }
-    out[h] = (T)(o * inv);
+    for (; s < S; ++s) o0 += wsu[s * stride + h] * s_w[s];
+    out[h] = (T)(((o0 + o1) + (o2 + o3)) * inv);
   }
 }
 
@@ -233,6 +270,9 @@ extern "C" int xmk_fmha_decode(const void* query, const void* key, const void* v
   p.scale2 = head_scale * kLog2e;
   const uint32_t units = num_batches * num_heads;
   plan(units, num_keys, &p.splits, &p.chunk);
+  if (p.splits > MAXSPLITS)
+    return xmk::fail(XMK_UNIMPLEMENTED, "fmha_decode: %u keys need %d splits, more than %d", num_keys, p.splits,
+                     MAXSPLITS);
   xmk::trace("fmha_decode B=%u N=%u T=%u H=%u splits=%d chunk=%d", num_batches, num_heads, num_keys,
              head_size, p.splits, p.chunk);
   if (dtype == XMK_BF16) launch<__bf16>(p, (int)units, (hipStream_t)stream);

@@ -10,17 +10,31 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // y = (x - mean) / sqrt(var + eps) * gamma + beta, one work-group per row, fp32 statistics.
-__global__ __launch_bounds__(256) void layernorm_kernel(const _Float16* __restrict__ x,
-                                                        const _Float16* __restrict__ gamma,
-                                                        const _Float16* __restrict__ beta,
-                                                        _Float16* __restrict__ y, int d, float eps) {
-  __shared__ float s_part[2][4];
+// A thread keeps its elements (8 per 16-byte load, up to LN_MAXV loads) in registers between the
+// statistics and the normalisation, so the row is read once.  d % 8 == 0, d <= 512 * 8 * LN_MAXV.
+constexpr int LN_NT = 512, LN_MAXV = 4;
+typedef uint32_t ln_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(LN_NT) void layernorm_kernel(const _Float16* __restrict__ x,
+                                                          const _Float16* __restrict__ gamma,
+                                                          const _Float16* __restrict__ beta,
+                                                          _Float16* __restrict__ y, int d, float eps) {
+  __shared__ float s_part[2][LN_NT / 64];
+  union Pack { ln_u32x4 u; _Float16 e[8]; };
   const _Float16* xr = x + (size_t)blockIdx.x * d;
+  Pack v[LN_MAXV];
   float s = 0.f, ss = 0.f;
-  for (int i = threadIdx.x; i < d; i += 256) {
-    const float v = (float)xr[i];
-    s += v;
-    ss += v * v;
+#pragma unroll
+  for (int j = 0; j < LN_MAXV; ++j) {
+    const int i = (threadIdx.x + j * LN_NT) * 8;
+    if (i < d) {
+      v[j].u = *reinterpret_cast<const ln_u32x4*>(xr + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = (float)v[j].e[e];
+        s += f;
+        ss += f * f;
+      }
+    }
   }
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) {
@@ -32,13 +46,29 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const _Float16* __restri
     s_part[1][threadIdx.x >> 6] = ss;
   }
   __syncthreads();
-  s = s_part[0][0] + s_part[0][1] + s_part[0][2] + s_part[0][3];
-  ss = s_part[1][0] + s_part[1][1] + s_part[1][2] + s_part[1][3];
+  s = 0.f;
+  ss = 0.f;
+#pragma unroll
+  for (int w = 0; w < LN_NT / 64; ++w) {
+    s += s_part[0][w];
+    ss += s_part[1][w];
+  }
   const float mean = s / d;
   const float var = fmaxf(ss / d - mean * mean, 0.f);
   const float rstd = rsqrtf(var + eps);
-  for (int i = threadIdx.x; i < d; i += 256)
-    y[(size_t)blockIdx.x * d + i] = (_Float16)(((float)xr[i] - mean) * rstd * (float)gamma[i] + (float)beta[i]);
+#pragma unroll
+  for (int j = 0; j < LN_MAXV; ++j) {
+    const int i = (threadIdx.x + j * LN_NT) * 8;
+    if (i < d) {
+      Pack g, b, o;
+      g.u = *reinterpret_cast<const ln_u32x4*>(gamma + i);
+      b.u = *reinterpret_cast<const ln_u32x4*>(beta + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        o.e[e] = (_Float16)(((float)v[j].e[e] - mean) * rstd * (float)g.e[e] + (float)b.e[e]);
+      *reinterpret_cast<ln_u32x4*>(y + (size_t)blockIdx.x * d + i) = o.u;
+    }
+  }
 }
 
 // qkv [B, 3 d] (columns q | k | v, head-major).  Rotates the first rotary_dim dims of every q
@@ -119,6 +149,8 @@ int check_cfg(const xmk_gptj_config* c) {
     return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: d_model != n_head * head_dim");
   if (c->head_dim % 8 != 0 || c->head_dim > 256 || c->rotary_dim % 2 != 0 || c->rotary_dim > c->head_dim)
     return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: unsupported head_dim / rotary_dim");
+  if (c->d_model > LN_NT * 8 * LN_MAXV)
+    return xmk::fail(XMK_UNIMPLEMENTED, "gptj_decode: d_model %d above %d", c->d_model, LN_NT * 8 * LN_MAXV);
   return XMK_OK;
 }
 
@@ -149,6 +181,8 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
   if (position < 0 || position >= cfg->cache_capacity)
     return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: position %d outside the cache (capacity %d)",
                      position, cfg->cache_capacity);
+  if (!xmk::aligned(hidden_in, 16) || !xmk::aligned(lnf_gamma, 16) || !xmk::aligned(lnf_beta, 16))
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: hidden_in and LayerNorm parameters must be 16-byte aligned");
   if (!xmk::aligned(workspace, 256)) return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: workspace must be 256-byte aligned");
   const xmk_gptj_config& c = *cfg;
   const Workspace w = carve(c, (char*)workspace);
@@ -165,7 +199,9 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
     const xmk_gptj_layer& L = layers[l];
     if (!L.ln_gamma || !L.ln_beta || !L.k_cache || !L.v_cache)
       return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: layer %d has a null pointer", l);
-    hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(256), 0, st, x, (const _Float16*)L.ln_gamma,
+    if (!xmk::aligned(L.ln_gamma, 16) || !xmk::aligned(L.ln_beta, 16))
+      return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: layer %d LayerNorm parameters must be 16-byte aligned", l);
+    hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(LN_NT), 0, st, x, (const _Float16*)L.ln_gamma,
                        (const _Float16*)L.ln_beta, w.h, (int)d, c.ln_eps);
     if ((rc = linear(L.qkv, w.h, w.qkv, B, d, 3 * d, c.group, xmk::Int4Epilogue{}, st, "qkv")) != XMK_OK) return rc;
     hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)c.n_head, (unsigned)B), dim3(256), 0, st, w.qkv, w.q,
@@ -190,7 +226,7 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
     x = xn;
     xn = (xn == w.x0) ? w.x1 : w.x0;
   }
-  hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(256), 0, st, x, (const _Float16*)lnf_gamma,
+  hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(LN_NT), 0, st, x, (const _Float16*)lnf_gamma,
                      (const _Float16*)lnf_beta, w.h, (int)d, c.ln_eps);
   if ((rc = linear(*lm_head, w.h, logits, B, d, c.vocab, c.group, xmk::Int4Epilogue{}, st, "lm_head")) != XMK_OK) return rc;
   return xmk::check_launch("gptj_decode");
