@@ -12,12 +12,21 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // y = (x - mean) / sqrt(var + eps) * gamma + beta, one work-group per row, fp32 statistics.
 // A thread keeps its elements (8 per 16-byte load, up to LN_MAXV loads) in registers between the
 // statistics and the normalisation, so the row is read once.  d % 8 == 0, d <= 512 * 8 * LN_MAXV.
+// With x_out != NULL the row is first assembled from the previous block's pieces,
+//     x = fp16( x_in + sum_s p1[s] + sum_s p2[s] + bias2 )
+// (p1, p2: fp32 partial sums [ks][32][d] of the K-split out_proj and fc_out GEMMs, added in slice
+// order), written to x_out, and normalised from the rounded value.
 constexpr int LN_NT = 512, LN_MAXV = 4;
 typedef uint32_t ln_u32x4 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(LN_NT) void layernorm_kernel(const _Float16* __restrict__ x,
                                                           const _Float16* __restrict__ gamma,
                                                           const _Float16* __restrict__ beta,
-                                                          _Float16* __restrict__ y, int d, float eps) {
+                                                          _Float16* __restrict__ y, int d, float eps,
+                                                          const float* __restrict__ p1, int ks1,
+                                                          const float* __restrict__ p2, int ks2,
+                                                          const _Float16* __restrict__ bias2,
+                                                          _Float16* __restrict__ x_out) {
+  typedef float ln_f32x4 __attribute__((ext_vector_type(4)));
   __shared__ float s_part[2][LN_NT / 64];
   union Pack { ln_u32x4 u; _Float16 e[8]; };
   const _Float16* xr = x + (size_t)blockIdx.x * d;
@@ -28,6 +37,30 @@ __global__ __launch_bounds__(LN_NT) void layernorm_kernel(const _Float16* __rest
     const int i = (threadIdx.x + j * LN_NT) * 8;
     if (i < d) {
       v[j].u = *reinterpret_cast<const ln_u32x4*>(xr + i);
+      if (x_out) {
+        float f[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = (float)v[j].e[e];
+        auto add_slices = [&](const float* p, int ks) {
+          for (int sl = 0; sl < ks; ++sl) {
+            const float* q = p + ((size_t)sl * 32 + blockIdx.x) * d + i;
+            const ln_f32x4 lo = *reinterpret_cast<const ln_f32x4*>(q), hi = *reinterpret_cast<const ln_f32x4*>(q + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { f[e] += lo[e]; f[4 + e] += hi[e]; }
+          }
+        };
+        add_slices(p1, ks1);
+        add_slices(p2, ks2);
+        if (bias2) {
+          Pack b2;
+          b2.u = *reinterpret_cast<const ln_u32x4*>(bias2 + i);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) f[e] += (float)b2.e[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[j].e[e] = (_Float16)f[e];
+        *reinterpret_cast<ln_u32x4*>(x_out + (size_t)blockIdx.x * d + i) = v[j].u;
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float f = (float)v[j].e[e];
@@ -112,6 +145,9 @@ struct Workspace {
   _Float16 *x0, *x1, *h, *qkv, *q, *attn, *ff;
   void* attn_ws;
   size_t attn_ws_bytes;
+  int ks_out, ks_fc;     // K slices of out_proj and fc_out (both 1: not split)
+  float *p_out, *p_fc;   // their partial sums
+  size_t p_bytes;
   size_t total;
 };
 
@@ -136,6 +172,13 @@ Workspace carve(const xmk_gptj_config& c, char* base) {
   w.attn_ws_bytes = xmk_fmha_decode_workspace_bytes((uint32_t)c.batch, (uint32_t)c.n_head,
                                                     (uint32_t)c.head_dim, (uint32_t)c.cache_capacity);
   w.attn_ws = take(w.attn_ws_bytes);
+  // fp32 partial sums of the K-split out_proj and fc_out GEMMs (when the plan splits them)
+  w.ks_out = xmk::int4_plan_split(c.batch, c.d_model, c.d_model, c.group);
+  w.ks_fc = xmk::int4_plan_split(c.batch, c.d_ff, c.d_model, c.group);
+  if (w.ks_out < 2 || w.ks_fc < 2) w.ks_out = w.ks_fc = 1;
+  w.p_bytes = (size_t)xmk::kInt4MaxSplit * 32 * d * sizeof(float);
+  w.p_out = (float*)take(w.p_bytes);
+  w.p_fc = (float*)take(w.p_bytes);
   w.total = off;
   return w;
 }
@@ -155,11 +198,12 @@ int check_cfg(const xmk_gptj_config* c) {
 }
 
 int linear(const xmk_int4_linear& l, const void* act, void* out, int64_t m, int64_t k, int64_t n,
-           int64_t group, const xmk::Int4Epilogue& ep, hipStream_t st, const char* what) {
+           int64_t group, const xmk::Int4Epilogue& ep, hipStream_t st, const char* what,
+           const xmk::Int4SplitK& split = xmk::Int4SplitK{}) {
   if (l.k != k || l.n != n)
     return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: %s is %lldx%lld, expected %lldx%lld", what,
                      (long long)l.k, (long long)l.n, (long long)k, (long long)n);
-  return xmk::int4_gemm_launch(act, l.qweight, l.scales, l.zeros, l.bias, out, m, k, n, group, ep, st);
+  return xmk::int4_gemm_launch(act, l.qweight, l.scales, l.zeros, l.bias, out, m, k, n, group, ep, st, split);
 }
 
 }  // namespace
@@ -193,16 +237,34 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
   const float scale = 1.0f / sqrtf((float)c.head_dim);
   const int64_t head_stride = (int64_t)c.cache_capacity * c.head_dim;
 
+  // With out_proj and fc_out split over K, a block ends with x (its input) and two sets of
+  // partial sums; the next LayerNorm assembles x' = x + out_proj(attn) + fc_out(...) + bias from
+  // them.  Otherwise fc_out's epilogue does (out_proj's result rounded to fp16 in between).
   const _Float16* x = (const _Float16*)hidden_in;
   _Float16* xn = w.x0;
+  const _Float16* pending_bias = nullptr;
+  bool pending = false;
+  auto run_ln = [&](const void* gamma, const void* beta) {
+    if (pending) {
+      hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(LN_NT), 0, st, x, (const _Float16*)gamma,
+                         (const _Float16*)beta, w.h, (int)d, c.ln_eps, (const float*)w.p_out, w.ks_out,
+                         (const float*)w.p_fc, w.ks_fc, pending_bias, xn);
+      x = xn;
+      xn = (xn == w.x0) ? w.x1 : w.x0;
+      pending = false;
+    } else {
+      hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(LN_NT), 0, st, x, (const _Float16*)gamma,
+                         (const _Float16*)beta, w.h, (int)d, c.ln_eps, (const float*)nullptr, 0, (const float*)nullptr,
+                         0, (const _Float16*)nullptr, (_Float16*)nullptr);
+    }
+  };
   for (int l = 0; l < c.n_layer; ++l) {
     const xmk_gptj_layer& L = layers[l];
     if (!L.ln_gamma || !L.ln_beta || !L.k_cache || !L.v_cache)
       return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: layer %d has a null pointer", l);
-    if (!xmk::aligned(L.ln_gamma, 16) || !xmk::aligned(L.ln_beta, 16))
-      return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: layer %d LayerNorm parameters must be 16-byte aligned", l);
-    hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(LN_NT), 0, st, x, (const _Float16*)L.ln_gamma,
-                       (const _Float16*)L.ln_beta, w.h, (int)d, c.ln_eps);
+    if (!xmk::aligned(L.ln_gamma, 16) || !xmk::aligned(L.ln_beta, 16) || !xmk::aligned(L.fc_out.bias, 16))
+      return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: layer %d LayerNorm parameters and fc_out bias must be 16-byte aligned", l);
+    run_ln(L.ln_gamma, L.ln_beta);
     if ((rc = linear(L.qkv, w.h, w.qkv, B, d, 3 * d, c.group, xmk::Int4Epilogue{}, st, "qkv")) != XMK_OK) return rc;
     hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)c.n_head, (unsigned)B), dim3(256), 0, st, w.qkv, w.q,
                        (_Float16*)L.k_cache, (_Float16*)L.v_cache, c.n_head, c.head_dim, c.rotary_dim,
@@ -211,23 +273,32 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
                               (uint32_t)c.head_dim, (uint32_t)(position + 1), head_stride, scale, w.attn_ws,
                               w.attn_ws_bytes, stream)) != XMK_OK)
       return rc;
-    // fc_in (+bias, gelu_new) from the same ln_1 output; fc_out adds bias, the residual x and the
-    // attention branch in its epilogue:  x' = x + out_proj(attn) + fc_out(...)
+    // fc_in (+bias, gelu_new) from the same ln_1 output
     xmk::Int4Epilogue gelu;
     gelu.gelu = 1;
     if ((rc = linear(L.fc_in, w.h, w.ff, B, d, dff, c.group, gelu, st, "fc_in")) != XMK_OK) return rc;
-    // out_proj result goes to w.qkv's first B*d elements (qkv is dead after the rotary kernel)
-    _Float16* a_out = w.qkv;
-    if ((rc = linear(L.out_proj, w.attn, a_out, B, d, d, c.group, xmk::Int4Epilogue{}, st, "out_proj")) != XMK_OK) return rc;
-    xmk::Int4Epilogue res;
-    res.add0 = x;
-    res.add1 = a_out;
-    if ((rc = linear(L.fc_out, w.ff, xn, B, dff, d, c.group, res, st, "fc_out")) != XMK_OK) return rc;
-    x = xn;
-    xn = (xn == w.x0) ? w.x1 : w.x0;
+    if (w.ks_out > 1 && !L.out_proj.bias) {  // (a biased out_proj takes the epilogue path)
+      xmk::Int4SplitK so, sf;
+      so.ksplit = w.ks_out; so.partial = w.p_out; so.partial_bytes = w.p_bytes;
+      sf.ksplit = w.ks_fc;  sf.partial = w.p_fc;  sf.partial_bytes = w.p_bytes;
+      if ((rc = linear(L.out_proj, w.attn, nullptr, B, d, d, c.group, xmk::Int4Epilogue{}, st, "out_proj", so)) != XMK_OK) return rc;
+      if ((rc = linear(L.fc_out, w.ff, nullptr, B, dff, d, c.group, xmk::Int4Epilogue{}, st, "fc_out", sf)) != XMK_OK) return rc;
+      pending = true;
+      pending_bias = (const _Float16*)L.fc_out.bias;
+    } else {
+      // out_proj result goes to w.qkv's first B*d elements (qkv is dead after the rotary kernel);
+      // fc_out adds bias, the residual x and the attention branch in its epilogue
+      _Float16* a_out = w.qkv;
+      if ((rc = linear(L.out_proj, w.attn, a_out, B, d, d, c.group, xmk::Int4Epilogue{}, st, "out_proj")) != XMK_OK) return rc;
+      xmk::Int4Epilogue res;
+      res.add0 = x;
+      res.add1 = a_out;
+      if ((rc = linear(L.fc_out, w.ff, xn, B, dff, d, c.group, res, st, "fc_out")) != XMK_OK) return rc;
+      x = xn;
+      xn = (xn == w.x0) ? w.x1 : w.x0;
+    }
   }
-  hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)B), dim3(LN_NT), 0, st, x, (const _Float16*)lnf_gamma,
-                     (const _Float16*)lnf_beta, w.h, (int)d, c.ln_eps);
+  run_ln(lnf_gamma, lnf_beta);
   if ((rc = linear(*lm_head, w.h, logits, B, d, c.vocab, c.group, xmk::Int4Epilogue{}, st, "lm_head")) != XMK_OK) return rc;
   return xmk::check_launch("gptj_decode");
 }

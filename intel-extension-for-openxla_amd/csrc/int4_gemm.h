@@ -14,8 +14,20 @@ struct Int4Epilogue {
   const void* add1 = nullptr;
 };
 
+// Splitting K over work-groups, for shapes whose N alone gives too few of them.  With
+// ksplit > 1 the launch writes fp32 partial sums [ksplit][32 rows][n] to `partial` and nothing
+// else: no bias, no epilogue, `out` untouched.  The consumer adds the slices in index order.
+struct Int4SplitK {
+  int ksplit = 1;
+  float* partial = nullptr;
+  size_t partial_bytes = 0;
+};
+constexpr int kInt4MaxSplit = 8;
+// Number of K slices worth using for this shape (1: do not split).
+int int4_plan_split(int64_t m, int64_t k, int64_t n, int64_t group);
+
 int int4_gemm_launch(const void* act, const void* qweight, const void* scales, const void* zeros,
                      const void* bias, void* out, int64_t m, int64_t k, int64_t n, int64_t group,
-                     const Int4Epilogue& ep, hipStream_t st);
+                     const Int4Epilogue& ep, hipStream_t st, const Int4SplitK& split = Int4SplitK{});
 
 }  // namespace xmk

@@ -112,12 +112,15 @@ __device__ __forceinline__ float half_at(const Words<NWORDS>& r, int c) {
 // SPG  : 32-channel k-steps per quantisation group (group = 32*SPG)
 // NW   : waves per block; wave w takes groups w, w+NW, ... and the partial
 //        sums meet in LDS in a fixed order (deterministic result)
-template <int W, int MT, int RI, int SPG, int NW>
+// SK   : K is also split over gridDim.y work-groups; slice y writes its fp32 partial sums
+//        [32 rows][N] to partial + y * 32 * N and applies no epilogue (the consumer adds the
+//        slices in a fixed order)
+template <int W, int MT, int RI, int SPG, int NW, bool SK>
 __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
     const _Float16* __restrict__ act, const uint32_t* __restrict__ qw,
     const _Float16* __restrict__ scales, const _Float16* __restrict__ zeros,
     const _Float16* __restrict__ bias, _Float16* __restrict__ out, int m_base, int M, int K,
-    int N, xmk::Int4Epilogue ep) {
+    int N, xmk::Int4Epilogue ep, float* __restrict__ partial) {
   constexpr int NCOL = 16 * W;
   constexpr int ROWS = MT == 2 ? 32 : (RI == 4 ? 16 : RI);  // rows the block reduces
   __shared__ float red[NW][ROWS][NCOL];
@@ -222,14 +225,17 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
   };
 
   GroupData bufA, bufB;  // ping-pong: no register copies between iterations
-  int g = wave;
-  if (g < ngroups) fetch(g, bufA);
-  while (g < ngroups) {
-    if (g + NW < ngroups) fetch(g + NW, bufB);
+  // This work-group's share of the groups: all of them, or slice blockIdx.y of gridDim.y.
+  const int gper = SK ? (ngroups + (int)gridDim.y - 1) / (int)gridDim.y : ngroups;
+  const int gend = SK ? min(ngroups, ((int)blockIdx.y + 1) * gper) : ngroups;
+  int g = (SK ? (int)blockIdx.y * gper : 0) + wave;
+  if (g < gend) fetch(g, bufA);
+  while (g < gend) {
+    if (g + NW < gend) fetch(g + NW, bufB);
     compute(bufA);
     g += NW;
-    if (g >= ngroups) break;
-    if (g + NW < ngroups) fetch(g + NW, bufA);
+    if (g >= gend) break;
+    if (g + NW < gend) fetch(g + NW, bufA);
     compute(bufB);
     g += NW;
   }
@@ -246,6 +252,20 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
   __syncthreads();
 
   const int rows = min(ROWS, M - m_base);
+  if constexpr (SK) {
+    // This work-group's partial sums, fp32, no epilogue: the consumer adds the slices up.
+    float* mine = partial + (size_t)blockIdx.y * 32 * N;
+    for (int e = threadIdx.x; e < rows * NCOL; e += NW * 64) {
+      const int row = e / NCOL, col = e % NCOL;
+      const int n = blockIdx.x * NCOL + col;
+      if (n >= N) continue;
+      float s = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) s += red[w][row][col];
+      mine[(size_t)row * N + n] = s;
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < rows * NCOL; e += NW * 64) {
     const int row = e / NCOL, col = e % NCOL;
     const int n = blockIdx.x * NCOL + col;
@@ -296,25 +316,40 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(
   }
 }
 
+struct SplitArgs {
+  int ksplit = 1;
+  float* partial = nullptr;
+};
+
 template <int W, int MT, int RI, int SPG, int NW>
 void launch(const void* act, const void* qw, const void* scales, const void* zeros,
             const void* bias, void* out, int m_base, int M, int K, int N,
-            const xmk::Int4Epilogue& ep, hipStream_t st) {
+            const xmk::Int4Epilogue& ep, hipStream_t st, const SplitArgs& sk) {
   const int blocks = (int)xmk::ceil_div(N, 16 * W);
-  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW>), dim3(blocks), dim3(NW * 64), 0, st,
+  if (sk.ksplit > 1) {
+    if constexpr (W == 4 && MT == 1) {  // the only shape the split is planned for
+      hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true>), dim3(blocks, sk.ksplit), dim3(NW * 64), 0, st,
+                         (const _Float16*)act, (const uint32_t*)qw, (const _Float16*)scales,
+                         (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N, ep,
+                         sk.partial);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false>), dim3(blocks), dim3(NW * 64), 0, st,
                      (const _Float16*)act, (const uint32_t*)qw, (const _Float16*)scales,
-                     (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N, ep);
+                     (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N, ep,
+                     (float*)nullptr);
 }
 
 template <int W, int MT, int RI, int NW>
 int launch_spg(int spg, const void* act, const void* qw, const void* scales, const void* zeros,
                const void* bias, void* out, int m_base, int M, int K, int N,
-               const xmk::Int4Epilogue& ep, hipStream_t st) {
+               const xmk::Int4Epilogue& ep, hipStream_t st, const SplitArgs& sk) {
   switch (spg) {
-    case 1: launch<W, MT, RI, 1, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
-    case 2: launch<W, MT, RI, 2, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
-    case 4: launch<W, MT, RI, 4, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
-    case 8: launch<W, MT, RI, 8, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st); break;
+    case 1: launch<W, MT, RI, 1, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
+    case 2: launch<W, MT, RI, 2, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
+    case 4: launch<W, MT, RI, 4, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
+    case 8: launch<W, MT, RI, 8, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
     default: return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   }
   return XMK_OK;
@@ -322,10 +357,29 @@ int launch_spg(int spg, const void* act, const void* qw, const void* scales, con
 
 }  // namespace
 
+int xmk::int4_plan_split(int64_t m, int64_t k, int64_t n, int64_t group) {
+  // Worth it when 64-column blocks alone cannot fill the device (256 CUs) and every wave of
+  // every slice still gets at least one quantisation group.
+  if (m > 16 || group <= 0 || k % group != 0) return 1;
+  const int64_t blocks = xmk::ceil_div(n, 64);
+  if (blocks >= 192) return 1;
+  // XMK_INT4_SPLIT=<k splits> overrides the choice (tuning aid).
+  static const char* split_env = getenv("XMK_INT4_SPLIT");
+  if (split_env) {
+    const int e = atoi(split_env);
+    if (e >= 1 && e <= kInt4MaxSplit) return e;
+  }
+  int ks = (int)(256 / blocks);
+  if (ks > kInt4MaxSplit) ks = kInt4MaxSplit;
+  while (ks > 1 && (k / group) / ks < 8) ks /= 2;
+  return ks < 1 ? 1 : ks;
+}
+
 int xmk::int4_gemm_launch(const void* act, const void* qweight, const void* scales,
                           const void* zeros, const void* bias, void* out, int64_t m, int64_t k,
-                          int64_t n, int64_t group, const Int4Epilogue& ep, hipStream_t st) {
-  if (!act || !qweight || !scales || !zeros || !out)
+                          int64_t n, int64_t group, const Int4Epilogue& ep, hipStream_t st,
+                          const Int4SplitK& split) {
+  if (!act || !qweight || !scales || !zeros || (!out && split.ksplit <= 1))
     return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: null pointer");
   if (m <= 0 || k <= 0 || n <= 0 || group <= 0)
     return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: non-positive size");
@@ -356,11 +410,22 @@ int xmk::int4_gemm_launch(const void* act, const void* qweight, const void* scal
       nw = enw;
     }
   }
-  xmk::trace("int4_gemm m=%d k=%d n=%d group=%d words_per_lane=%d waves=%d", M, K, N, (int)group, w, nw);
+  SplitArgs sk;
+  if (split.ksplit > 1) {
+    if (M > 16 || !split.partial || split.ksplit > kInt4MaxSplit ||
+        split.partial_bytes < (size_t)split.ksplit * 32 * N * sizeof(float))
+      return xmk::fail(XMK_INTERNAL, "int4_gemm: bad K split request");
+    w = 4;
+    nw = 8;
+    sk.ksplit = split.ksplit;
+    sk.partial = split.partial;
+  }
+  xmk::trace("int4_gemm m=%d k=%d n=%d group=%d words_per_lane=%d waves=%d ksplit=%d", M, K, N, (int)group, w, nw,
+             sk.ksplit);
   for (int m_base = 0; m_base < M; m_base += 32) {
     const int rows = M - m_base;
     int rc;
-#define XMK_INT4_ARGS spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st
+#define XMK_INT4_ARGS spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk
 #define XMK_INT4_CASE(WW)                                                   \
   do {                                                                      \
     if (rows > 16) rc = launch_spg<WW, 2, 4, 8>(XMK_INT4_ARGS);             \
