@@ -429,9 +429,7 @@ int xmk::int4_gemm_launch(const void* act, const void* qweight, const void* scal
 #define XMK_INT4_CASE(WW)                                                   \
   do {                                                                      \
     if (rows > 16) rc = launch_spg<WW, 2, 4, 8>(XMK_INT4_ARGS);             \
-    else if (rows > 4) rc = launch_spg<WW, 1, 4, 8>(XMK_INT4_ARGS);         \
-    else if (rows > 1) rc = nw == 16 ? launch_spg<WW, 1, 4, 16>(XMK_INT4_ARGS) \
-                                     : launch_spg<WW, 1, 4, 8>(XMK_INT4_ARGS); \
+    else if (rows > 1) rc = launch_spg<WW, 1, 4, 8>(XMK_INT4_ARGS);         \
     else rc = nw == 16 ? launch_spg<WW, 1, 1, 16>(XMK_INT4_ARGS)            \
                        : launch_spg<WW, 1, 1, 8>(XMK_INT4_ARGS);            \
   } while (0)
