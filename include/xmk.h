@@ -114,6 +114,16 @@ const char* xmk_last_error(void);
  * tiled kernel, where the reference falls back to oneDNN. */
 int xmk_gemm(const xmk_gemm_desc* desc, void* stream);
 
+/* Three GEMMs that share the left operand: out_i = act(lhs · rhs_i + bias_i), i = q, k, v.
+ * Replaces XetlaQKVGemmKernel (xetla/gemm/gemm.h:112-170) and hgemm_qkv / hgemm_qkv_bias
+ * (xetla/gemm/hgemm_impl.h:461-608), which the reference launches as one kernel over a
+ * 3 x tiles grid.  desc describes the first product: rhs.data is rhs_q and rhs.batch_stride
+ * the distance in elements to rhs_k and from there to rhs_v (k*n when the three weights are
+ * stacked, as the reference assumes, hgemm_impl.h:523-527); out.data is out_q, and out_k,
+ * out_v are laid out like it; bias, when the epilogue adds one, holds the three vectors
+ * stacked [3, n].  batch_size 1, beta 0, 16-bit dtype_in == dtype_out. */
+int xmk_gemm_qkv(const xmk_gemm_desc* desc, void* out_k, void* out_v, void* stream);
+
 /* Name of the tile policy xmk_gemm would pick for (m, n, k): the counterpart
  * of selectXetlaGemmConfig (xetla/gemm/gemm.cc:286-308).  Returns a static
  * string. */

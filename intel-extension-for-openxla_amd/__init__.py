@@ -121,6 +121,18 @@ def run_gemm(lhs, rhs, out, *, lhs_transpose=False, rhs_transpose=False, out_tra
     return out
 
 
+def run_gemm_qkv(lhs, weights, out_q, out_k, out_v, *, rhs_transpose=False, bias=None, epilogue=EPI_DEFAULT,
+                 stream=None):
+    """out_i = act(lhs @ weights[i] + bias[i]) for the three stacked weights [3, k, n] (or [3, n, k] with
+    ``rhs_transpose``) in one launch; bias is [3, n] or None."""
+    rhs = matrix(weights[0], rhs_transpose)
+    rhs.batch_stride = weights.stride(0)
+    d = GemmDesc(matrix(lhs, False), rhs, matrix(out_q, False), None,
+                 None if bias is None else bias.data_ptr(), dtype_code(lhs), dtype_code(out_q), 1, 1.0, 0.0, epilogue)
+    _check(lib().xmk_gemm_qkv(ctypes.byref(d), _ptr(out_k), _ptr(out_v), _stream(stream)))
+    return out_q, out_k, out_v
+
+
 def gemm_policy_name(m, n, k, rhs_transpose=False, dtype_in=BF16, dtype_out=BF16):
     return lib().xmk_gemm_policy_name(ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
                                       ctypes.c_int32(int(rhs_transpose)), ctypes.c_int32(dtype_in),

@@ -52,6 +52,8 @@ struct GenericParams {
   int kin, kout;
   float alpha, beta;
   int act;
+  void* out_alt[2];  // see GemmParams
+  int64_t sbias;
 };
 
 __global__ __launch_bounds__(256) void gemm_generic_kernel(GenericParams p) {
@@ -60,6 +62,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GenericParams p) {
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
   const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
   const int64_t bz = blockIdx.z;
+  if (p.out_alt[0] && bz > 0) p.out = p.out_alt[bz - 1];
   const bool integer = p.kin == G_S8;
   float acc[4][4] = {};
   int iacc[4][4] = {};
@@ -114,7 +117,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GenericParams p) {
       }
       float v = p.alpha * acc[i][j];
       if (p.beta != 0.f && p.c) v += p.beta * load_as_f32(p.c, p.kout, off);
-      if (p.bias) v += load_as_f32(p.bias, p.kin, n);
+      if (p.bias) v += load_as_f32(p.bias, p.kin, bz * p.sbias + n);
       v = apply_act(v, p.act);
       switch (p.kout) {
         case G_BF16: reinterpret_cast<__bf16*>(p.out)[off] = (__bf16)v; break;
@@ -157,7 +160,25 @@ extern "C" const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int
   return kPolicies[select_policy(m, n, k)].name;
 }
 
-extern "C" int xmk_gemm(const xmk_gemm_desc* d, void* stream) {
+namespace {
+// out1 / out2: further outputs of the shared-lhs three-GEMM form, or null for a plain GEMM.
+int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream);
+}  // namespace
+
+extern "C" int xmk_gemm(const xmk_gemm_desc* d, void* stream) { return run_gemm(d, nullptr, nullptr, stream); }
+
+extern "C" int xmk_gemm_qkv(const xmk_gemm_desc* d, void* out_k, void* out_v, void* stream) {
+  if (!d) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm_qkv: null descriptor");
+  if (!out_k || !out_v) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm_qkv: null output");
+  if (d->batch_size != 1 || d->beta != 0.0f || d->out.transpose)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gemm_qkv: needs batch_size 1, beta 0 and a row-major output");
+  if (d->dtype_in != d->dtype_out || (d->dtype_in != XMK_BF16 && d->dtype_in != XMK_F16))
+    return xmk::fail(XMK_UNIMPLEMENTED, "gemm_qkv: 16-bit input and output of one type only");  // gemm.h:112-170
+  return run_gemm(d, out_k, out_v, stream);
+}
+
+namespace {
+int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
   if (!d) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: null descriptor");
   if (!d->lhs.data || !d->rhs.data || !d->out.data)
     return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: null operand");
@@ -219,6 +240,7 @@ extern "C" int xmk_gemm(const xmk_gemm_desc* d, void* stream) {
   if (!d->bias && wants_bias) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: bias missing");
 
   hipStream_t st = (hipStream_t)stream;
+  const bool qkv = out1 != nullptr;
   const bool sixteen = din == XMK_BF16 || din == XMK_F16;
 #ifdef XMK_GEMM_MINIMAL  // tuning builds: one dtype, A row-major, largest tile only
   const bool minimal_ok = din == XMK_BF16 && dout == XMK_BF16 && !lhs.transpose && select_policy(m, n, k) == 0;
@@ -226,7 +248,8 @@ extern "C" int xmk_gemm(const xmk_gemm_desc* d, void* stream) {
   const bool minimal_ok = true;
 #endif
   const bool fast = minimal_ok && sixteen && xmk::aligned(lhs.data, 16) && xmk::aligned(rhs.data, 16) &&
-                    xmk::aligned(out.data, 16) && lhs.leading_dim_stride % 8 == 0 &&
+                    xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) && xmk::aligned(out2, 16) &&
+                    lhs.leading_dim_stride % 8 == 0 &&
                     rhs.leading_dim_stride % 8 == 0 && lhs.batch_stride % 8 == 0 &&
                     rhs.batch_stride % 8 == 0 && lhs.num_cols % 8 == 0 && rhs.num_cols % 8 == 0;
   if (fast) {
@@ -237,13 +260,15 @@ extern "C" int xmk_gemm(const xmk_gemm_desc* d, void* stream) {
     p.lda = lhs.leading_dim_stride; p.ldb = rhs.leading_dim_stride; p.ldc = out.leading_dim_stride;
     p.sa = lhs.batch_stride; p.sb = rhs.batch_stride; p.sc = out.batch_stride;
     p.alpha = d->alpha; p.beta = d->beta; p.act = act;
+    p.out_alt[0] = out1; p.out_alt[1] = out2; p.sbias = 0;
+    if (qkv) { p.sa = 0; p.sc = 0; p.sbias = n; }
     const bool a_mc = lhs.transpose != 0;   // stored [K, M]
     const bool b_mc = rhs.transpose == 0;   // stored [K, N]
     const int pol = select_policy(m, n, k);
     xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s",
                (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
                rhs.transpose, d->epilogue, d->beta, kPolicies[pol].name);
-    const int batch = (int)d->batch_size;
+    const int batch = qkv ? 3 : (int)d->batch_size;
 #ifdef XMK_GEMM_MINIMAL
     p.tiles_m = (int)xmk::ceil_div(p.M, 256);
     p.tiles_n = (int)xmk::ceil_div(p.N, 256);
@@ -281,10 +306,13 @@ extern "C" int xmk_gemm(const xmk_gemm_desc* d, void* stream) {
   g.ta = lhs.transpose; g.tb = rhs.transpose;
   g.kin = generic_kind(din); g.kout = generic_kind(dout);
   g.alpha = d->alpha; g.beta = d->beta; g.act = act;
+  g.out_alt[0] = out1; g.out_alt[1] = out2; g.sbias = 0;
+  if (qkv) { g.sa = 0; g.sc = 0; g.sbias = n; }
   xmk::trace("gemm m=%lld n=%lld k=%lld -> generic_64x64", (long long)m, (long long)n, (long long)k);
   hipLaunchKernelGGL(gemm_generic_kernel,
                      dim3((unsigned)xmk::ceil_div(n, 64), (unsigned)xmk::ceil_div(m, 64),
-                          (unsigned)d->batch_size),
+                          (unsigned)(qkv ? 3 : d->batch_size)),
                      dim3(256), 0, st, g);
   return xmk::check_launch("gemm");
 }
+}  // namespace

@@ -33,6 +33,10 @@ struct GemmParams {
   float alpha, beta;
   int act;
   int tiles_m, tiles_n;
+  // Shared-lhs multi-output form (three GEMMs with one A): batch member z > 0 writes to
+  // out_alt[z - 1] instead of out + z * sc and reads bias + z * sbias.  Null when unused.
+  void* out_alt[2];
+  int64_t sbias;
 };
 
 __device__ __forceinline__ float gelu_tanh(float x) {
@@ -442,6 +446,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   // Epilogue.  acc[i][j][e] is out[m][n] with m = m0 + wm WTM + 32 i + lane%32 and
   // n = n0 + wn WTN + 32 j + 8 (e/4) + 4 (lane/32) + e%4.
   const int64_t coff = bz * p.sc;
+  GemmParams q = p;  // this batch member's view of the output and bias
+  if (p.out_alt[0] && bz > 0) q.out = p.out_alt[bz - 1];
+  if (p.bias) q.bias = reinterpret_cast<const T*>(p.bias) + bz * p.sbias;
   static_for<TM>([&](auto I) {
     constexpr int i = decltype(I)::value;
     const int m = m0 + wm * WTM + i * 32 + (lane & 31);
@@ -449,10 +456,10 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
       constexpr int j = decltype(J)::value;
       const floatx16 t = acc[i][j];
       const int nb = n0 + wn * WTN + j * 32 + (lane >> 5) * 4;
-      store_quad<T, OutF32>(p, floatx4{t[0], t[1], t[2], t[3]}, m, nb, coff);
-      store_quad<T, OutF32>(p, floatx4{t[4], t[5], t[6], t[7]}, m, nb + 8, coff);
-      store_quad<T, OutF32>(p, floatx4{t[8], t[9], t[10], t[11]}, m, nb + 16, coff);
-      store_quad<T, OutF32>(p, floatx4{t[12], t[13], t[14], t[15]}, m, nb + 24, coff);
+      store_quad<T, OutF32>(q, floatx4{t[0], t[1], t[2], t[3]}, m, nb, coff);
+      store_quad<T, OutF32>(q, floatx4{t[4], t[5], t[6], t[7]}, m, nb + 8, coff);
+      store_quad<T, OutF32>(q, floatx4{t[8], t[9], t[10], t[11]}, m, nb + 16, coff);
+      store_quad<T, OutF32>(q, floatx4{t[12], t[13], t[14], t[15]}, m, nb + 24, coff);
     });
   });
 }

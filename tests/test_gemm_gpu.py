@@ -195,3 +195,33 @@ def test_errors(xmk):
     with pytest.raises(xmk.XmkError) as e:
         xmk.run_gemm(a, b, out.float().half())  # bf16 x bf16 -> f16 is not an accepted triple
     assert e.value.code == xmk.INTERNAL
+
+
+@pytest.mark.parametrize("dt_name", ["BF16", "F16"])
+@pytest.mark.parametrize("m,n,k,rhs_t,with_bias", [(4, 4096, 4096, False, False), (200, 264, 136, True, True),
+                                                   (512, 1024, 256, False, True), (33, 72, 100, False, False)])
+def test_qkv_fused_gemm(xmk, oracle, dt_name, m, n, k, rhs_t, with_bias):
+    """Three products sharing A in one launch (the reference's hgemm_qkv / hgemm_qkv_bias; its own
+    check is example/qkv_fusion/test_qkv_fusion.py: m=4, k=n=4096 fp16, fused vs separate)."""
+    dt = getattr(oracle, dt_name)
+    kind = _kind(dt, oracle)
+    tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+    a = oracle.from_f32(oracle.normal((m, k), 70, k ** -0.5), dt)
+    w = oracle.from_f32(oracle.normal((3, n, k) if rhs_t else (3, k, n), 71, 1.0), dt)
+    bias = oracle.from_f32(oracle.normal((3, n), 72, 0.5), dt) if with_bias else None
+    outs = [torch.full((m, n), float("nan"), dtype=tdt, device="cuda") for _ in range(3)]
+    xmk.run_gemm_qkv(to_dev(a, kind), to_dev(w, kind), *outs, rhs_transpose=rhs_t,
+                     bias=None if bias is None else to_dev(bias, kind),
+                     epilogue=xmk.EPI_BIAS if with_bias else xmk.EPI_DEFAULT)
+    torch.cuda.synchronize()
+    for i in range(3):
+        _, ref = oracle.gemm(a, w[i], dt, dt, rhs_t=rhs_t, bias=None if bias is None else bias[i],
+                             epilogue=oracle.EPI_BIAS if with_bias else oracle.EPI_DEFAULT)
+        _check(oracle, outs[i].float().cpu().numpy(), ref[0])
+    # fused == separate, bit for bit (same kernel, same tile order)
+    sep = torch.empty((m, n), dtype=tdt, device="cuda")
+    xmk.run_gemm(to_dev(a, kind), to_dev(w[1], kind), sep, rhs_transpose=rhs_t,
+                 bias=None if bias is None else to_dev(bias[1], kind),
+                 epilogue=xmk.EPI_BIAS if with_bias else xmk.EPI_DEFAULT)
+    torch.cuda.synchronize()
+    assert torch.equal(sep.view(torch.int16), outs[1].view(torch.int16))
