@@ -4,6 +4,7 @@
 #pragma once
 #include <hip/hip_bf16.h>
 
+#include <cstdlib>
 #include <utility>
 
 #include "common.h"
@@ -478,15 +479,41 @@ constexpr Policy kPolicies[] = {
 };
 constexpr int kNumPolicies = sizeof(kPolicies) / sizeof(kPolicies[0]);
 
-// Largest tile that still gives every CU of the device (256) work; the role of
-// selectXetlaGemmConfig (xetla/gemm/gemm.cc:286-308), without a per-shape table.
+// Tile choice, the role of selectXetlaGemmConfig (xetla/gemm/gemm.cc:286-308).  Shapes listed in the tuned table
+// (gemm_policy_table.h, written by autotune_gemm.py from measurements) take the policy
+// recorded there, as the reference's configMap does (gemm.cc:31-285).
+// XMK_GEMM_POLICY=<index> forces one policy for every shape (what the autotuner uses).
+struct TunedShape {
+  int m, n, k, policy;
+};
+#include "gemm_policy_table.h"
 inline int select_policy(int64_t m, int64_t n, int64_t k) {
-  (void)k;
+  static const int forced = [] {
+    const char* e = getenv("XMK_GEMM_POLICY");
+    const int v = e ? atoi(e) : -1;
+    return (e && v >= 0 && v < kNumPolicies) ? v : -1;
+  }();
+  if (forced >= 0) return forced;
+  for (const TunedShape& t : kTunedShapes)
+    if (t.m == m && t.n == n && t.k == k) return t.policy;
+  // Heuristic: the policy with the best estimated throughput = (what the tile sustains when the
+  // device is full) x (share of the 256 CUs busy over the tile waves) x (share of the tiles' area
+  // inside the matrix).  The per-tile figures are measured large-shape rates relative to 256x256.
+  static constexpr float kTileRate[kNumPolicies] = {1.0f, 0.75f, 0.60f, 0.55f};
+  int best = kNumPolicies - 1;
+  float best_score = -1.0f;
   for (int i = 0; i < kNumPolicies; ++i) {
     const int64_t tiles = xmk::ceil_div(m, kPolicies[i].bm) * xmk::ceil_div(n, kPolicies[i].bn);
-    if (tiles >= 256 || i == kNumPolicies - 1) return i;
+    const int64_t waves = xmk::ceil_div(tiles, 256);
+    const float busy = (float)tiles / (float)(waves * 256);
+    const float inside = (float)((double)m * (double)n / ((double)tiles * kPolicies[i].bm * kPolicies[i].bn));
+    const float score = kTileRate[i] * busy * inside;
+    if (score > best_score) {
+      best = i;
+      best_score = score;
+    }
   }
-  return kNumPolicies - 1;
+  return best;
 }
 
 template <typename T, bool OutF32, bool A_MC, bool B_MC, int BM, int BN, int WGM, int WGN, int BK, int NSTAGE>
