@@ -147,6 +147,25 @@ int xmk_fmha_fwd(const void* query, const void* key, const void* value, const vo
                  uint32_t num_heads, uint32_t head_size, uint32_t num_queries,
                  uint32_t num_keys, float head_scale, int32_t causal, void* stream);
 
+/* Bytes of device workspace xmk_fmha_bwd needs for the given shape. */
+size_t xmk_fmha_bwd_workspace_bytes(uint32_t num_batches, uint32_t num_heads, uint32_t head_size,
+                                    uint32_t num_queries, uint32_t num_keys);
+
+/* Fused multi-head-attention backward.  Replaces fmha_backward_kernel_fp16 / _bf16
+ * (xetla/sdp/sdp_backward.h:22-36; same tensors, with the reference's two scratch arguments
+ * dp_sum and grad_query_accum folded into one workspace, the dtype and `causal` as arguments).
+ *   query, key, value, bias, out as in xmk_fmha_fwd; grad_out [B,N,F,H]; lse fp32 [B*N,F] as
+ *   written by xmk_fmha_fwd; grad_query [B,N,F,H], grad_key and grad_value [B,N,T,H] of dtype.
+ * No gradient is produced for the bias (the reference passes d_bias but never writes it,
+ * xetla_gpu_fused_mha_runner.cc:383-385).  workspace: 256-byte aligned device memory of at least
+ * xmk_fmha_bwd_workspace_bytes() bytes. */
+int xmk_fmha_bwd(const void* query, const void* key, const void* value, const void* bias,
+                 const void* out, const void* grad_out, const float* lse, void* grad_query,
+                 void* grad_key, void* grad_value, int32_t dtype, uint32_t num_batches,
+                 uint32_t num_heads, uint32_t head_size, uint32_t num_queries, uint32_t num_keys,
+                 float head_scale, int32_t causal, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
 /* Bytes of device workspace xmk_fmha_decode needs for the given shape. */
 size_t xmk_fmha_decode_workspace_bytes(uint32_t num_batches, uint32_t num_heads,
                                        uint32_t head_size, uint32_t num_keys);

@@ -65,7 +65,8 @@ def lib():
         for name, restype in (("xmk_version", ctypes.c_char_p),
                               ("xmk_last_error", ctypes.c_char_p),
                               ("xmk_gemm_policy_name", ctypes.c_char_p),
-                              ("xmk_fmha_decode_workspace_bytes", ctypes.c_size_t)):
+                              ("xmk_fmha_decode_workspace_bytes", ctypes.c_size_t),
+                              ("xmk_fmha_bwd_workspace_bytes", ctypes.c_size_t)):
             if hasattr(L, name):
                 getattr(L, name).restype = restype
         _lib = L
@@ -152,6 +153,23 @@ def fmha_forward(query, key, value, out, *, bias=None, lse=None, head_scale=None
                               ctypes.c_uint32(T), ctypes.c_float(scale),
                               ctypes.c_int32(int(causal)), _stream(stream)))
     return out
+
+
+def fmha_backward(query, key, value, out, grad_out, lse, *, bias=None, head_scale=None, causal=False, stream=None):
+    """Gradients (dq, dk, dv) of fmha_forward's output with respect to query, key, value."""
+    B, N, F, H = query.shape
+    T = key.shape[2]
+    scale = (H ** -0.5) if head_scale is None else head_scale
+    nbytes = lib().xmk_fmha_bwd_workspace_bytes(ctypes.c_uint32(B), ctypes.c_uint32(N), ctypes.c_uint32(H),
+                                                ctypes.c_uint32(F), ctypes.c_uint32(T))
+    ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=query.device)
+    dq, dk, dv = torch.empty_like(query), torch.empty_like(key), torch.empty_like(value)
+    _check(lib().xmk_fmha_bwd(_ptr(query), _ptr(key), _ptr(value), _ptr(bias), _ptr(out), _ptr(grad_out), _ptr(lse),
+                              _ptr(dq), _ptr(dk), _ptr(dv), ctypes.c_int32(dtype_code(query)), ctypes.c_uint32(B),
+                              ctypes.c_uint32(N), ctypes.c_uint32(H), ctypes.c_uint32(F), ctypes.c_uint32(T),
+                              ctypes.c_float(scale), ctypes.c_int32(int(causal)), _ptr(ws), ctypes.c_size_t(nbytes),
+                              _stream(stream)))
+    return dq, dk, dv
 
 
 def fmha_decode_workspace_bytes(B, N, H, T):

@@ -250,6 +250,28 @@ def fmha_fwd_online(q, k, v, dtype, scale, *, bias=None, causal=False, kBc=128):
     return out_f32
 
 
+def fmha_bwd(q, k, v, d_out, dtype, scale, *, bias=None, causal=False):
+    """Gradients of softmax(scale q k^T + bias + mask) v with respect to q, k, v, in float64 from the
+    rounded inputs (numpy; for test sizes).  The closed form the reference's backward kernel follows
+    (xetla/sdp/fmha_backward.h): P = softmax(S); dV = P^T dO; dP = dO V^T;
+    dS = P o (dP - rowsum(dP o P)); dQ = scale dS K; dK = scale dS^T Q.  Returns (dq, dk, dv) float64."""
+    qf, kf, vf, gf = (to_f32(x, dtype).astype(np.float64) for x in (q, k, v, d_out))
+    s = scale * np.einsum("bnfh,bnth->bnft", qf, kf)
+    if bias is not None:
+        s = s + to_f32(bias, dtype).astype(np.float64)
+    F, T = s.shape[-2:]
+    if causal:
+        s = np.where(np.arange(T)[None, :] > np.arange(F)[:, None], -np.inf, s)
+    p = np.exp(s - s.max(axis=-1, keepdims=True))
+    p /= p.sum(axis=-1, keepdims=True)
+    dv = np.einsum("bnft,bnfh->bnth", p, gf)
+    dp = np.einsum("bnfh,bnth->bnft", gf, vf)
+    ds = p * (dp - (dp * p).sum(axis=-1, keepdims=True))
+    dq = scale * np.einsum("bnft,bnth->bnfh", ds, kf)
+    dk = scale * np.einsum("bnft,bnfh->bnth", ds, qf)
+    return dq, dk, dv
+
+
 def num_threads():
     return int(lib().xo_num_threads())
 

@@ -1,0 +1,72 @@
+"""GPU parity: fused attention backward through the C ABI (xmk_fmha_bwd) against the oracle's
+float64 closed form (pinned by finite differences in tests/test_oracle_math.py).
+
+Tolerance: error relative to the tensor's scale (oracle.rel_err's first figure) <= 1e-2 as for the
+forward outputs; the elementwise figure <= 1e-2 for fp16 and <= 5e-2 for bf16.  P, dS and the
+forward output O (which enters through D = rowsum(dO o O)) are rounded to the 16-bit operand type
+before the products that consume them, here as in the reference (xetla/sdp/fmha_backward.h:195-196);
+the measured elementwise error is rounding-dominated: <= 0.35 % for fp16 and eight times that
+(three mantissa bits fewer) for bf16.  The reference's own attention test allows atol 3e-2 for
+bf16 and 1e-2 for fp16 on O(1) outputs (test/jax_ut.patch:997)."""
+import numpy as np
+import pytest
+import torch
+
+from util import to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+TOL_ELEM = {"bf16": 5e-2, "fp16": 1e-2}
+
+
+def _run(xmk, oracle, name, B, N, F, T, H, causal, use_bias, seed=0, tol_elem=None):
+    dt = oracle.BF16 if name == "bf16" else oracle.F16
+    tdt = torch.bfloat16 if name == "bf16" else torch.float16
+    q = oracle.from_f32(oracle.normal((B, N, F, H), seed + 1), dt)
+    k = oracle.from_f32(oracle.normal((B, N, T, H), seed + 2), dt)
+    v = oracle.from_f32(oracle.normal((B, N, T, H), seed + 3), dt)
+    g = oracle.from_f32(oracle.normal((B, N, F, H), seed + 4), dt)
+    bias = oracle.from_f32(oracle.normal((B, N, F, T), seed + 5), dt) if use_bias else None
+    scale = H ** -0.5
+    dq, dk, dv = oracle.fmha_bwd(q, k, v, g, dt, scale, bias=bias, causal=causal)
+    kind = "bf16" if name == "bf16" else "f16"
+    tq, tk, tv, tg = (to_dev(x, kind) for x in (q, k, v, g))
+    tb = None if bias is None else to_dev(bias, kind)
+    out = torch.empty_like(tq)
+    lse = torch.empty((B * N, F), dtype=torch.float32, device="cuda")
+    xmk.fmha_forward(tq, tk, tv, out, bias=tb, lse=lse, causal=causal)
+    gq, gk, gv = xmk.fmha_backward(tq, tk, tv, out, tg, lse, bias=tb, causal=causal)
+    torch.cuda.synchronize()
+    errs = {}
+    for nm, got, ref in (("dq", gq, dq), ("dk", gk, dk), ("dv", gv, dv)):
+        ge, ee = oracle.rel_err(got.float().cpu().numpy(), ref.astype(np.float32))
+        errs[nm] = (ge, ee)
+        assert ge <= TOL and ee <= (tol_elem or TOL_ELEM[name]), (nm, ge, ee)
+    return errs
+
+
+@pytest.mark.parametrize("name", ["bf16", "fp16"])
+@pytest.mark.parametrize("causal,use_bias", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("F,T,H", [(128, 128, 64), (200, 136, 128), (64, 77, 40), (257, 64, 256)])
+def test_backward_shapes(xmk, oracle, name, causal, use_bias, F, T, H):
+    _run(xmk, oracle, name, 2, 3, F, T, H, causal, use_bias)
+
+
+def test_backward_chunks_over_units(xmk, oracle):
+    """More units than fit one workspace chunk (score buffers are capped at 1 GiB).  The maximum
+    over 1.5 M elements of a rounding-dominated error sits further out in the tail than on the
+    small shapes, so the elementwise bound is wider here; the scale-relative bound is the same."""
+    errs = _run(xmk, oracle, "bf16", 1, 12, 2048, 2048, 64, True, False, seed=9, tol_elem=1e-1)
+    print(errs)
+
+
+def test_backward_errors(xmk):
+    q = torch.zeros((1, 1, 8, 64), dtype=torch.float16, device="cuda")
+    lse = torch.zeros((1, 8), dtype=torch.float32, device="cuda")
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.fmha_backward(q.float(), q.float(), q.float(), q.float(), q.float(), lse)
+    assert e.value.code == xmk.INTERNAL and "Invalid MHA datatype" in e.value.message
+    q2 = torch.zeros((1, 1, 8, 60), dtype=torch.float16, device="cuda")
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.fmha_backward(q2, q2, q2, q2, q2, lse)
+    assert e.value.code == xmk.UNIMPLEMENTED

@@ -238,3 +238,45 @@ def test_fmha_online_form_agrees(oracle, causal):
     online = oracle.fmha_fwd_online(q, k, v, dt, H ** -0.5, causal=causal, kBc=32)
     assert np.abs(online - closed).max() < 3e-2
     assert oracle.rel_err(online, closed)[0] < 1e-2
+
+
+@pytest.mark.parametrize("causal,use_bias", [(False, False), (True, True)])
+def test_fmha_bwd_matches_finite_differences(oracle, causal, use_bias):
+    """The backward closed form against central differences of the forward closed form (float64,
+    fp16-exact inputs so that the rounding in from_f32 is the identity)."""
+    rng = np.random.default_rng(3)
+    B, N, F, T, H = 1, 2, 5, 7, 8
+    scale = 0.37
+
+    def r(shape):
+        return (rng.integers(-8, 9, size=shape) / 8.0).astype(np.float32)  # exact in fp16
+    q, k, v, g = r((B, N, F, H)), r((B, N, T, H)), r((B, N, T, H)), r((B, N, F, H))
+    bias = r((B, N, F, T)) if use_bias else None
+
+    def fwd(q_, k_, v_):
+        s = scale * np.einsum("bnfh,bnth->bnft", q_, k_)
+        if bias is not None:
+            s = s + bias
+        if causal:
+            s = np.where(np.arange(T)[None, :] > np.arange(F)[:, None], -np.inf, s)
+        p = np.exp(s - s.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        return np.einsum("bnft,bnth->bnfh", p, v_)
+
+    bits = lambda x: oracle.from_f32(x, oracle.F16)
+    dq, dk, dv = oracle.fmha_bwd(bits(q), bits(k), bits(v), bits(g), oracle.F16, scale,
+                                 bias=None if bias is None else bits(bias), causal=causal)
+    eps = 1e-5
+    for name, x, grad in (("q", q, dq), ("k", k, dk), ("v", v, dv)):
+        num = np.zeros(x.shape)
+        xd = x.astype(np.float64)
+        for idx in np.ndindex(*x.shape):
+            xp, xm = xd.copy(), xd.copy()
+            xp[idx] += eps
+            xm[idx] -= eps
+            args_p = [q.astype(np.float64), k.astype(np.float64), v.astype(np.float64)]
+            args_m = list(args_p)
+            i = "qkv".index(name)
+            args_p[i], args_m[i] = xp, xm
+            num[idx] = ((fwd(*args_p) - fwd(*args_m)) * g).sum() / (2 * eps)
+        assert np.abs(num - grad).max() <= 1e-6 * max(1.0, np.abs(grad).max()), name
