@@ -130,6 +130,7 @@ struct Loader {
   uint32_t sstride;  // bytes between consecutive loads of this wave (uniform)
   int kin0;          // k (inside the K step) of this lane's chunk in load 0
   bool ok[NL];       // this lane's row / column exists
+  uint32_t okoff[NL];  // ok[i] ? voff : kOob -- the offset of load i in a K step that lies fully inside K
 
   __device__ __forceinline__ void init(int64_t ld, int valid, int wave, int lane) {
     const int lrow = wave * RPL + lane / CPR;  // LDS row in load 0: operand row (KC) or k (MC)
@@ -145,13 +146,17 @@ struct Loader {
 #pragma unroll
       for (int i = 0; i < NL; ++i) ok[i] = chunk * 8 < valid;
     }
+#pragma unroll
+    for (int i = 0; i < NL; ++i) okoff[i] = ok[i] ? voff : kOob;
   }
   // Issues load i.  base: address of the tile origin for this K step; kleft: k of the step that
   // exist (<= 0 past the end of K: every lane is then out of range and the load writes zeros).
+  // CHECK_K = false: the caller knows that the whole K step exists (kleft >= BK).
+  template <bool CHECK_K = true>
   __device__ __forceinline__ void issue_one(int i, __amdgpu_buffer_rsrc_t rsrc, int kleft, char* lds_tile,
                                             int wave) const {
     const int k = MC ? kin0 + i * LSTRIDE : kin0;
-    const uint32_t off = (ok[i] && k < kleft) ? voff : kOob;
+    const uint32_t off = CHECK_K ? ((ok[i] && k < kleft) ? voff : kOob) : okoff[i];
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)(lds_tile + (i * NWAVES + wave) * 1024), 16,
                                              off, i * sstride, 0, 0);
   }
@@ -397,7 +402,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   // before the barrier, all but the youngest (NSTAGE-2) steps' loads of this wave have landed
   // (loads return in order), so step kt + 1 is complete once every wave has arrived, and this
   // wave's reads of `cur` are done, so `cur` may be overwritten by the loads the next step issues.
-  auto k_step = [&](const char* __restrict__ cur, const char* __restrict__ nxt, char* __restrict__ wr, int kt) {
+  auto k_step = [&](auto CHECK, const char* __restrict__ cur, const char* __restrict__ nxt, char* __restrict__ wr,
+                    int kt) {
+    constexpr bool CHECK_K = decltype(CHECK)::value;
     TSTAMP(0);
     const int kleft = p.K - (kt + NSTAGE - 1) * BK;
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(a_tile), rb = make_rsrc(b_tile);
@@ -420,9 +427,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
 #endif
       }
 #pragma unroll
-      for (int i = la0; i < la1; ++i) la.issue_one(i, ra, kleft, wr, wave);
+      for (int i = la0; i < la1; ++i) la.template issue_one<CHECK_K>(i, ra, kleft, wr, wave);
 #pragma unroll
-      for (int i = lb0; i < lb1; ++i) lb.issue_one(i, rb, kleft, wr + A_BYTES, wave);
+      for (int i = lb0; i < lb1; ++i) lb.template issue_one<CHECK_K>(i, rb, kleft, wr + A_BYTES, wave);
       if constexpr (ks + 1 < KS) read_frags(cur, ks + 1, (ks + 1) & 1);
       else read_frags(nxt, 0, KS & 1);
       mma(ks & 1);
@@ -439,8 +446,16 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   static_assert(KS % 2 == 0, "fragment double-buffering assumes an even number of k-steps");
   static_assert(NSTAGE >= 3, "the barrier leaves the running step's loads in flight");
   read_frags(lds, 0, 0);
-  for (int kt = 0; kt < KT; ++kt)
-    k_step(lds + (kt % NSTAGE) * STAGE, lds + ((kt + 1) % NSTAGE) * STAGE,
+  // Step kt loads K step kt + NSTAGE - 1: all of it exists until that index reaches the last
+  // (possibly partial) step, so only the final NSTAGE - 1 iterations (and a partial last K step)
+  // need the per-lane K test.
+  const int kt_full = min(KT, p.K / BK - (NSTAGE - 1));
+  int kt = 0;
+  for (; kt < kt_full; ++kt)
+    k_step(std::false_type{}, lds + (kt % NSTAGE) * STAGE, lds + ((kt + 1) % NSTAGE) * STAGE,
+           lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE, kt);
+  for (; kt < KT; ++kt)
+    k_step(std::true_type{}, lds + (kt % NSTAGE) * STAGE, lds + ((kt + 1) % NSTAGE) * STAGE,
            lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE, kt);
   __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));  // drain the zero-fill loads before LDS is released
 
