@@ -242,12 +242,7 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   const bool qkv = out1 != nullptr;
   const bool sixteen = din == XMK_BF16 || din == XMK_F16;
-#ifdef XMK_GEMM_MINIMAL  // tuning builds: one dtype, A row-major, largest tile only
-  const bool minimal_ok = din == XMK_BF16 && dout == XMK_BF16 && !lhs.transpose && select_policy(m, n, k) == 0;
-#else
-  const bool minimal_ok = true;
-#endif
-  const bool fast = minimal_ok && sixteen && xmk::aligned(lhs.data, 16) && xmk::aligned(rhs.data, 16) &&
+  const bool fast = sixteen && xmk::aligned(lhs.data, 16) && xmk::aligned(rhs.data, 16) &&
                     xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) && xmk::aligned(out2, 16) &&
                     lhs.leading_dim_stride % 8 == 0 &&
                     rhs.leading_dim_stride % 8 == 0 && lhs.batch_stride % 8 == 0 &&
@@ -269,21 +264,6 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
                (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
                rhs.transpose, d->epilogue, d->beta, kPolicies[pol].name);
     const int batch = qkv ? 3 : (int)d->batch_size;
-#ifdef XMK_GEMM_MINIMAL
-    p.tiles_m = (int)xmk::ceil_div(p.M, 256);
-    p.tiles_n = (int)xmk::ceil_div(p.N, 256);
-#ifndef XMK_EXP_CFG
-#define XMK_EXP_CFG 256, 256, 2, 2, 32, 4
-#endif
-#ifndef XMK_EXP_BM
-#define XMK_EXP_BM 256
-#define XMK_EXP_BN 256
-#endif
-    p.tiles_m = (int)xmk::ceil_div(p.M, XMK_EXP_BM);
-    p.tiles_n = (int)xmk::ceil_div(p.N, XMK_EXP_BN);
-    if (b_mc) launch_mfma<__bf16, false, false, true, XMK_EXP_CFG>(p, batch, st);
-    else launch_mfma<__bf16, false, false, false, XMK_EXP_CFG>(p, batch, st);
-#else
     if (din == XMK_BF16) {
       if (dout == XMK_F32) launch_layout<__bf16, true>(a_mc, b_mc, pol, p, batch, st);
       else launch_layout<__bf16, false>(a_mc, b_mc, pol, p, batch, st);
@@ -291,7 +271,6 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
       if (dout == XMK_F32) launch_layout<_Float16, true>(a_mc, b_mc, pol, p, batch, st);
       else launch_layout<_Float16, false>(a_mc, b_mc, pol, p, batch, st);
     }
-#endif
     return xmk::check_launch("gemm");
   }
 

@@ -347,10 +347,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   for (int st = 0; st < NSTAGE - 1; ++st) {
     la.issue(a_tile, p.K - st * BK, lds + st * STAGE, wave);
     lb.issue(b_tile, p.K - st * BK, lds + st * STAGE + A_BYTES, wave);
-#ifndef XMK_EXP_NOADVANCE
     a_tile += a_step;
     b_tile += b_step;
-#endif
   }
   __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 2) * LOADS));  // step 0 has landed (loads return in order)
   __builtin_amdgcn_s_barrier();
@@ -388,13 +386,6 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
         __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);               // 1 VMEM read
     }
   };
-#ifdef XMK_EXP_TIMING
-  long long* tlog = reinterpret_cast<long long*>(const_cast<void*>(p.bias));
-  const bool tl = blockIdx.x == 0 && tid == 0 && tlog != nullptr;
-#define TSTAMP(i) do { if (tl && kt < 16) tlog[kt * 8 + (i)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define TSTAMP(i)
-#endif
   // One K step: compute from stage `cur`, prefetch the first fragments of stage `nxt`, and fill
   // stage `wr` with K step kt + NSTAGE - 1.  The three stages are distinct; saying so
   // (__restrict__) lets the compiler keep the LDS-DMA loads in flight across the fragment reads
@@ -405,7 +396,6 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   auto k_step = [&](auto CHECK, const char* __restrict__ cur, const char* __restrict__ nxt, char* __restrict__ wr,
                     int kt) {
     constexpr bool CHECK_K = decltype(CHECK)::value;
-    TSTAMP(0);
     const int kleft = p.K - (kt + NSTAGE - 1) * BK;
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(a_tile), rb = make_rsrc(b_tile);
     static_for<KS>([&](auto KSI) {
@@ -414,17 +404,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
       constexpr int la0 = LoaderA::NL * ks / KS, la1 = LoaderA::NL * (ks + 1) / KS;
       constexpr int lb0 = LoaderB::NL * ks / KS, lb1 = LoaderB::NL * (ks + 1) / KS;
       if constexpr (ks + 1 == KS) {
-        TSTAMP(1);
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 3) * LOADS + LoaderA::NL * ks / KS + LoaderB::NL * ks / KS) &
                                    ~(0xf << 8));  // and lgkmcnt(0)
-        TSTAMP(2);
         __builtin_amdgcn_s_barrier();
-        TSTAMP(3);
-#ifdef XMK_EXP_STAGGER
-        // The waves leave the barrier together and run identical instruction streams; a small
-        // wave-dependent delay keeps their loads from queueing at the CU's one address unit.
-        for (int d = 0; d < wave; ++d) asm volatile("s_nop %0" ::"n"(XMK_EXP_STAGGER));
-#endif
       }
 #pragma unroll
       for (int i = la0; i < la1; ++i) la.template issue_one<CHECK_K>(i, ra, kleft, wr, wave);
@@ -436,11 +418,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
       interleave((la1 - la0) + (lb1 - lb0));
       __builtin_amdgcn_sched_barrier(0);
     });
-#ifndef XMK_EXP_NOADVANCE
     a_tile += a_step;
     b_tile += b_step;
-#endif
-    TSTAMP(4);
   };
 
   static_assert(KS % 2 == 0, "fragment double-buffering assumes an even number of k-steps");
@@ -537,7 +516,6 @@ void launch_mfma(const GemmParams& p, int batch, hipStream_t st) {
                      dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WGM * WGN * 64), 0, st, p);
 }
 
-#ifndef XMK_GEMM_MINIMAL
 template <typename T, bool OutF32, bool A_MC, bool B_MC>
 void launch_policy(int pol, GemmParams& p, int batch, hipStream_t st) {
   p.tiles_m = (int)xmk::ceil_div(p.M, kPolicies[pol].bm);
@@ -557,7 +535,6 @@ void launch_layout_impl(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch,
   else if (a_mc && !b_mc) launch_policy<T, OutF32, true, false>(pol, p, batch, st);
   else launch_policy<T, OutF32, true, true>(pol, p, batch, st);
 }
-#endif
 
 
 // Explicitly instantiated in gemm_inst_*.hip.
