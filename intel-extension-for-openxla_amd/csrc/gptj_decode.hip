@@ -197,13 +197,15 @@ int check_cfg(const xmk_gptj_config* c) {
   return XMK_OK;
 }
 
-int linear(const xmk_int4_linear& l, const void* act, void* out, int64_t m, int64_t k, int64_t n,
-           int64_t group, const xmk::Int4Epilogue& ep, hipStream_t st, const char* what,
-           const xmk::Int4SplitK& split = xmk::Int4SplitK{}) {
+// One int4 linear of the block as a launchable product.
+int make_call(const xmk_int4_linear& l, const void* act, void* out, int64_t k, int64_t n, const xmk::Int4Epilogue& ep,
+              const char* what, xmk::Int4Call* c, const xmk::Int4SplitK& split = xmk::Int4SplitK{}) {
   if (l.k != k || l.n != n)
     return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: %s is %lldx%lld, expected %lldx%lld", what,
                      (long long)l.k, (long long)l.n, (long long)k, (long long)n);
-  return xmk::int4_gemm_launch(act, l.qweight, l.scales, l.zeros, l.bias, out, m, k, n, group, ep, st, split);
+  c->act = act; c->qweight = l.qweight; c->scales = l.scales; c->zeros = l.zeros; c->bias = l.bias; c->out = out;
+  c->k = k; c->n = n; c->ep = ep; c->split = split;
+  return XMK_OK;
 }
 
 }  // namespace
@@ -265,7 +267,13 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
     if (!xmk::aligned(L.ln_gamma, 16) || !xmk::aligned(L.ln_beta, 16) || !xmk::aligned(L.fc_out.bias, 16))
       return xmk::fail(XMK_INVALID_ARGUMENT, "gptj_decode: layer %d LayerNorm parameters and fc_out bias must be 16-byte aligned", l);
     run_ln(L.ln_gamma, L.ln_beta);
-    if ((rc = linear(L.qkv, w.h, w.qkv, B, d, 3 * d, c.group, xmk::Int4Epilogue{}, st, "qkv")) != XMK_OK) return rc;
+    // q/k/v and fc_in (+bias, gelu_new) read the same ln_1 output: one launch carries both.
+    xmk::Int4Epilogue gelu;
+    gelu.gelu = 1;
+    xmk::Int4Call c_qkv, c_fc_in, c_out, c_fc_out;
+    if ((rc = make_call(L.qkv, w.h, w.qkv, d, 3 * d, xmk::Int4Epilogue{}, "qkv", &c_qkv)) != XMK_OK) return rc;
+    if ((rc = make_call(L.fc_in, w.h, w.ff, d, dff, gelu, "fc_in", &c_fc_in)) != XMK_OK) return rc;
+    if ((rc = xmk::int4_gemm_launch2(c_qkv, &c_fc_in, B, c.group, st)) != XMK_OK) return rc;
     hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)c.n_head, (unsigned)B), dim3(256), 0, st, w.qkv, w.q,
                        (_Float16*)L.k_cache, (_Float16*)L.v_cache, c.n_head, c.head_dim, c.rotary_dim,
                        c.cache_capacity, position);
@@ -273,32 +281,35 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
                               (uint32_t)c.head_dim, (uint32_t)(position + 1), head_stride, scale, w.attn_ws,
                               w.attn_ws_bytes, stream)) != XMK_OK)
       return rc;
-    // fc_in (+bias, gelu_new) from the same ln_1 output
-    xmk::Int4Epilogue gelu;
-    gelu.gelu = 1;
-    if ((rc = linear(L.fc_in, w.h, w.ff, B, d, dff, c.group, gelu, st, "fc_in")) != XMK_OK) return rc;
     if (w.ks_out > 1 && !L.out_proj.bias) {  // (a biased out_proj takes the epilogue path)
+      // out_proj(attn) and fc_out(ff) are independent: one launch, K split over work-groups, fp32
+      // partial sums that the next LayerNorm adds up.
       xmk::Int4SplitK so, sf;
       so.ksplit = w.ks_out; so.partial = w.p_out; so.partial_bytes = w.p_bytes;
       sf.ksplit = w.ks_fc;  sf.partial = w.p_fc;  sf.partial_bytes = w.p_bytes;
-      if ((rc = linear(L.out_proj, w.attn, nullptr, B, d, d, c.group, xmk::Int4Epilogue{}, st, "out_proj", so)) != XMK_OK) return rc;
-      if ((rc = linear(L.fc_out, w.ff, nullptr, B, dff, d, c.group, xmk::Int4Epilogue{}, st, "fc_out", sf)) != XMK_OK) return rc;
+      if ((rc = make_call(L.out_proj, w.attn, nullptr, d, d, xmk::Int4Epilogue{}, "out_proj", &c_out, so)) != XMK_OK) return rc;
+      if ((rc = make_call(L.fc_out, w.ff, nullptr, dff, d, xmk::Int4Epilogue{}, "fc_out", &c_fc_out, sf)) != XMK_OK) return rc;
+      if ((rc = xmk::int4_gemm_launch2(c_out, &c_fc_out, B, c.group, st)) != XMK_OK) return rc;
       pending = true;
       pending_bias = (const _Float16*)L.fc_out.bias;
     } else {
       // out_proj result goes to w.qkv's first B*d elements (qkv is dead after the rotary kernel);
       // fc_out adds bias, the residual x and the attention branch in its epilogue
       _Float16* a_out = w.qkv;
-      if ((rc = linear(L.out_proj, w.attn, a_out, B, d, d, c.group, xmk::Int4Epilogue{}, st, "out_proj")) != XMK_OK) return rc;
+      if ((rc = make_call(L.out_proj, w.attn, a_out, d, d, xmk::Int4Epilogue{}, "out_proj", &c_out)) != XMK_OK) return rc;
+      if ((rc = xmk::int4_gemm_launch2(c_out, nullptr, B, c.group, st)) != XMK_OK) return rc;
       xmk::Int4Epilogue res;
       res.add0 = x;
       res.add1 = a_out;
-      if ((rc = linear(L.fc_out, w.ff, xn, B, dff, d, c.group, res, st, "fc_out")) != XMK_OK) return rc;
+      if ((rc = make_call(L.fc_out, w.ff, xn, dff, d, res, "fc_out", &c_fc_out)) != XMK_OK) return rc;
+      if ((rc = xmk::int4_gemm_launch2(c_fc_out, nullptr, B, c.group, st)) != XMK_OK) return rc;
       x = xn;
       xn = (xn == w.x0) ? w.x1 : w.x0;
     }
   }
   run_ln(lnf_gamma, lnf_beta);
-  if ((rc = linear(*lm_head, w.h, logits, B, d, c.vocab, c.group, xmk::Int4Epilogue{}, st, "lm_head")) != XMK_OK) return rc;
+  xmk::Int4Call c_head;
+  if ((rc = make_call(*lm_head, w.h, logits, d, c.vocab, xmk::Int4Epilogue{}, "lm_head", &c_head)) != XMK_OK) return rc;
+  if ((rc = xmk::int4_gemm_launch2(c_head, nullptr, B, c.group, st)) != XMK_OK) return rc;
   return xmk::check_launch("gptj_decode");
 }

@@ -26,6 +26,22 @@ constexpr int kInt4MaxSplit = 8;
 // Number of K slices worth using for this shape (1: do not split).
 int int4_plan_split(int64_t m, int64_t k, int64_t n, int64_t group);
 
+// One product out = epilogue(act [m, k] x dequant(qweight) [k, n] + bias), or its K-split partial sums.
+struct Int4Call {
+  const void* act = nullptr;
+  const void* qweight = nullptr;
+  const void* scales = nullptr;
+  const void* zeros = nullptr;
+  const void* bias = nullptr;
+  void* out = nullptr;
+  int64_t k = 0, n = 0;
+  Int4Epilogue ep;
+  Int4SplitK split;
+};
+// Launches `a` and, if non-null, the independent product `b` (same m and group size): in one
+// grid when both take the same tile shape, else one after the other.
+int int4_gemm_launch2(const Int4Call& a, const Int4Call* b, int64_t m, int64_t group, hipStream_t st);
+
 int int4_gemm_launch(const void* act, const void* qweight, const void* scales, const void* zeros,
                      const void* bias, void* out, int64_t m, int64_t k, int64_t n, int64_t group,
                      const Int4Epilogue& ep, hipStream_t st, const Int4SplitK& split = Int4SplitK{});

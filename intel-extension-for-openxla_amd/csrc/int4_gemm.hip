@@ -115,12 +115,36 @@ __device__ __forceinline__ float half_at(const Words<NWORDS>& r, int c) {
 // SK   : K is also split over gridDim.y work-groups; slice y writes its fp32 partial sums
 //        [32 rows][N] to partial + y * 32 * N and applies no epilogue (the consumer adds the
 //        slices in a fixed order)
+//
+// One launch can carry two independent products of the same tile shape (e.g. the q/k/v and
+// fc_in projections of a decoder block, which read the same activations): blocks
+// [0, blocks0) work on p0, the rest on p1.
+struct Int4Problem {
+  const _Float16* act;
+  const uint32_t* qw;
+  const _Float16* scales;
+  const _Float16* zeros;
+  const _Float16* bias;
+  _Float16* out;
+  int m_base, M, K, N;
+  xmk::Int4Epilogue ep;
+  float* partial;
+};
+
 template <int W, int MT, int RI, int SPG, int NW, bool SK>
-__global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
-    const _Float16* __restrict__ act, const uint32_t* __restrict__ qw,
-    const _Float16* __restrict__ scales, const _Float16* __restrict__ zeros,
-    const _Float16* __restrict__ bias, _Float16* __restrict__ out, int m_base, int M, int K,
-    int N, xmk::Int4Epilogue ep, float* __restrict__ partial) {
+__global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0) {
+  const bool second = (int)blockIdx.x >= blocks0;
+  const int bx = (int)blockIdx.x - (second ? blocks0 : 0);
+  const _Float16* __restrict__ act = second ? p1.act : p0.act;
+  const uint32_t* __restrict__ qw = second ? p1.qw : p0.qw;
+  const _Float16* __restrict__ scales = second ? p1.scales : p0.scales;
+  const _Float16* __restrict__ zeros = second ? p1.zeros : p0.zeros;
+  const _Float16* __restrict__ bias = second ? p1.bias : p0.bias;
+  _Float16* __restrict__ out = second ? p1.out : p0.out;
+  const int m_base = second ? p1.m_base : p0.m_base, M = second ? p1.M : p0.M;
+  const int K = second ? p1.K : p0.K, N = second ? p1.N : p0.N;
+  const xmk::Int4Epilogue ep = second ? p1.ep : p0.ep;
+  float* __restrict__ partial = second ? p1.partial : p0.partial;
   constexpr int NCOL = 16 * W;
   constexpr int ROWS = MT == 2 ? 32 : (RI == 4 ? 16 : RI);  // rows the block reduces
   __shared__ float red[NW][ROWS][NCOL];
@@ -129,7 +153,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
   const int kg = lane >> 4;
-  const int n0 = blockIdx.x * NCOL + col16 * W;
+  const int n0 = bx * NCOL + col16 * W;
   const bool col_ok = n0 < N;
   const int ngroups = K / (32 * SPG);
 
@@ -257,7 +281,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
     float* mine = partial + (size_t)blockIdx.y * 32 * N;
     for (int e = threadIdx.x; e < rows * NCOL; e += NW * 64) {
       const int row = e / NCOL, col = e % NCOL;
-      const int n = blockIdx.x * NCOL + col;
+      const int n = bx * NCOL + col;
       if (n >= N) continue;
       float s = 0.f;
 #pragma unroll
@@ -268,7 +292,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(
   }
   for (int e = threadIdx.x; e < rows * NCOL; e += NW * 64) {
     const int row = e / NCOL, col = e % NCOL;
-    const int n = blockIdx.x * NCOL + col;
+    const int n = bx * NCOL + col;
     if (n >= N) continue;
     float s = 0.f;
 #pragma unroll
@@ -316,43 +340,118 @@ __global__ __launch_bounds__(256) void int4_dequant_kernel(
   }
 }
 
-struct SplitArgs {
-  int ksplit = 1;
-  float* partial = nullptr;
+// One product as the host sees it, and the tile configuration chosen for it.
+struct Config {
+  int w = 4, nw = 16, ksplit = 1;
+  bool operator==(const Config& o) const { return w == o.w && nw == o.nw && ksplit == o.ksplit; }
 };
 
 template <int W, int MT, int RI, int SPG, int NW>
-void launch(const void* act, const void* qw, const void* scales, const void* zeros,
-            const void* bias, void* out, int m_base, int M, int K, int N,
-            const xmk::Int4Epilogue& ep, hipStream_t st, const SplitArgs& sk) {
-  const int blocks = (int)xmk::ceil_div(N, 16 * W);
-  if (sk.ksplit > 1) {
+void launch(const Int4Problem& a, const Int4Problem* b, int ksplit, hipStream_t st) {
+  const int blocks0 = (int)xmk::ceil_div(a.N, 16 * W);
+  const int blocks = blocks0 + (b ? (int)xmk::ceil_div(b->N, 16 * W) : 0);
+  const Int4Problem& second = b ? *b : a;
+  if (ksplit > 1) {
     if constexpr (W == 4 && MT == 1) {  // the only shape the split is planned for
-      hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true>), dim3(blocks, sk.ksplit), dim3(NW * 64), 0, st,
-                         (const _Float16*)act, (const uint32_t*)qw, (const _Float16*)scales,
-                         (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N, ep,
-                         sk.partial);
+      hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true>), dim3(blocks, ksplit), dim3(NW * 64), 0, st, a,
+                         second, blocks0);
       return;
     }
   }
-  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false>), dim3(blocks), dim3(NW * 64), 0, st,
-                     (const _Float16*)act, (const uint32_t*)qw, (const _Float16*)scales,
-                     (const _Float16*)zeros, (const _Float16*)bias, (_Float16*)out, m_base, M, K, N, ep,
-                     (float*)nullptr);
+  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false>), dim3(blocks), dim3(NW * 64), 0, st, a, second,
+                     blocks0);
 }
 
 template <int W, int MT, int RI, int NW>
-int launch_spg(int spg, const void* act, const void* qw, const void* scales, const void* zeros,
-               const void* bias, void* out, int m_base, int M, int K, int N,
-               const xmk::Int4Epilogue& ep, hipStream_t st, const SplitArgs& sk) {
+int launch_spg(int spg, const Int4Problem& a, const Int4Problem* b, int ksplit, hipStream_t st) {
   switch (spg) {
-    case 1: launch<W, MT, RI, 1, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
-    case 2: launch<W, MT, RI, 2, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
-    case 4: launch<W, MT, RI, 4, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
-    case 8: launch<W, MT, RI, 8, NW>(act, qw, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk); break;
+    case 1: launch<W, MT, RI, 1, NW>(a, b, ksplit, st); break;
+    case 2: launch<W, MT, RI, 2, NW>(a, b, ksplit, st); break;
+    case 4: launch<W, MT, RI, 4, NW>(a, b, ksplit, st); break;
+    case 8: launch<W, MT, RI, 8, NW>(a, b, ksplit, st); break;
     default: return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   }
   return XMK_OK;
+}
+
+// Checks one product and picks its tile configuration.
+int prepare(const xmk::Int4Call& c, int64_t m, int64_t group, Config* cfg) {
+  if (!c.act || !c.qweight || !c.scales || !c.zeros || (!c.out && c.split.ksplit <= 1))
+    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: null pointer");
+  const int64_t k = c.k, n = c.n;
+  if (m <= 0 || k <= 0 || n <= 0 || group <= 0)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: non-positive size");
+  if (n % 8 != 0 || group % 8 != 0 || k % group != 0)
+    return xmk::fail(XMK_INVALID_ARGUMENT,
+                     "int4_gemm: need n %% 8 == 0, group %% 8 == 0, k %% group == 0 (m=%lld k=%lld "
+                     "n=%lld group=%lld)", (long long)m, (long long)k, (long long)n, (long long)group);
+  if (group % 32 != 0 || group > 256)
+    return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
+  if (k > (1 << 24) || n > (1 << 24) || m > (1 << 24))
+    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: dimension too large");
+  if (!xmk::aligned(c.act, 16) || !xmk::aligned(c.qweight, 16) || !xmk::aligned(c.scales, 8) ||
+      !xmk::aligned(c.zeros, 8) || !xmk::aligned(c.out, 2))
+    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: act, qweight must be 16-byte and scales, zeros 8-byte aligned");
+  // Words per lane: the widest load that still yields about one block per CU.
+  cfg->w = 4;
+  if (n / 64 < 192) cfg->w = 2;
+  if (n / 32 < 192) cfg->w = 1;
+  cfg->nw = 16;
+  // XMK_INT4_TILE="<words per lane>,<waves per block>" overrides the choice (tuning aid).
+  static const char* tile_env = getenv("XMK_INT4_TILE");
+  if (tile_env) {
+    int ew = 0, enw = 0;
+    if (sscanf(tile_env, "%d,%d", &ew, &enw) == 2 && (ew == 1 || ew == 2 || ew == 4) && (enw == 8 || enw == 16)) {
+      cfg->w = ew;
+      cfg->nw = enw;
+    }
+  }
+  cfg->ksplit = 1;
+  if (c.split.ksplit > 1) {
+    if (m > 16 || !c.split.partial || c.split.ksplit > xmk::kInt4MaxSplit ||
+        c.split.partial_bytes < (size_t)c.split.ksplit * 32 * n * sizeof(float))
+      return xmk::fail(XMK_INTERNAL, "int4_gemm: bad K split request");
+    cfg->w = 4;
+    cfg->nw = 8;
+    cfg->ksplit = c.split.ksplit;
+  }
+  return XMK_OK;
+}
+
+Int4Problem problem(const xmk::Int4Call& c, int m_base, int M) {
+  Int4Problem p;
+  p.act = (const _Float16*)c.act; p.qw = (const uint32_t*)c.qweight; p.scales = (const _Float16*)c.scales;
+  p.zeros = (const _Float16*)c.zeros; p.bias = (const _Float16*)c.bias; p.out = (_Float16*)c.out;
+  p.m_base = m_base; p.M = M; p.K = (int)c.k; p.N = (int)c.n;
+  p.ep = c.ep;
+  p.partial = c.split.ksplit > 1 ? c.split.partial : nullptr;
+  return p;
+}
+
+// Launches `a` (and `b`, if given, in the same grid) for rows [m_base, m_base + 32).
+int launch_cfg(const Config& cfg, int spg, const xmk::Int4Call& a, const xmk::Int4Call* b, int m_base, int M,
+               hipStream_t st) {
+  const Int4Problem pa = problem(a, m_base, M);
+  Int4Problem pb_store;
+  const Int4Problem* pb = nullptr;
+  if (b) {
+    pb_store = problem(*b, m_base, M);
+    pb = &pb_store;
+  }
+  const int rows = M - m_base;
+  int rc;
+#define XMK_INT4_CASE(WW)                                                            \
+  do {                                                                               \
+    if (rows > 16) rc = launch_spg<WW, 2, 4, 8>(spg, pa, pb, cfg.ksplit, st);        \
+    else if (rows > 1) rc = launch_spg<WW, 1, 4, 8>(spg, pa, pb, cfg.ksplit, st);    \
+    else rc = cfg.nw == 16 ? launch_spg<WW, 1, 1, 16>(spg, pa, pb, cfg.ksplit, st)   \
+                           : launch_spg<WW, 1, 1, 8>(spg, pa, pb, cfg.ksplit, st);   \
+  } while (0)
+  if (cfg.w == 4) XMK_INT4_CASE(4);
+  else if (cfg.w == 2) XMK_INT4_CASE(2);
+  else XMK_INT4_CASE(1);
+#undef XMK_INT4_CASE
+  return rc;
 }
 
 }  // namespace
@@ -375,72 +474,32 @@ int xmk::int4_plan_split(int64_t m, int64_t k, int64_t n, int64_t group) {
   return ks < 1 ? 1 : ks;
 }
 
+int xmk::int4_gemm_launch2(const Int4Call& a, const Int4Call* b, int64_t m, int64_t group, hipStream_t st) {
+  Config ca, cb;
+  int rc = prepare(a, m, group, &ca);
+  if (rc != XMK_OK) return rc;
+  if (b && (rc = prepare(*b, m, group, &cb)) != XMK_OK) return rc;
+  const int spg = (int)(group / 32);
+  const int M = (int)m;
+  // One grid for both when they take the same tile shape; else one after the other.
+  const bool together = b && ca == cb;
+  xmk::trace("int4_gemm m=%d k=%lld n=%lld group=%d words_per_lane=%d waves=%d ksplit=%d%s", M, (long long)a.k,
+             (long long)a.n, (int)group, ca.w, ca.nw, ca.ksplit, together ? " (+ a second product in the same launch)" : "");
+  for (int m_base = 0; m_base < M; m_base += 32) {
+    if ((rc = launch_cfg(ca, spg, a, together ? b : nullptr, m_base, M, st)) != XMK_OK) return rc;
+    if (b && !together && (rc = launch_cfg(cb, spg, *b, nullptr, m_base, M, st)) != XMK_OK) return rc;
+  }
+  return xmk::check_launch("int4_gemm");
+}
+
 int xmk::int4_gemm_launch(const void* act, const void* qweight, const void* scales,
                           const void* zeros, const void* bias, void* out, int64_t m, int64_t k,
                           int64_t n, int64_t group, const Int4Epilogue& ep, hipStream_t st,
                           const Int4SplitK& split) {
-  if (!act || !qweight || !scales || !zeros || (!out && split.ksplit <= 1))
-    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: null pointer");
-  if (m <= 0 || k <= 0 || n <= 0 || group <= 0)
-    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: non-positive size");
-  if (n % 8 != 0 || group % 8 != 0 || k % group != 0)
-    return xmk::fail(XMK_INVALID_ARGUMENT,
-                     "int4_gemm: need n %% 8 == 0, group %% 8 == 0, k %% group == 0 (m=%lld k=%lld "
-                     "n=%lld group=%lld)", (long long)m, (long long)k, (long long)n, (long long)group);
-  if (group % 32 != 0 || group > 256)
-    return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
-  if (k > (1 << 24) || n > (1 << 24) || m > (1 << 24))
-    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: dimension too large");
-  if (!xmk::aligned(act, 16) || !xmk::aligned(qweight, 16) || !xmk::aligned(scales, 8) || !xmk::aligned(zeros, 8) ||
-      !xmk::aligned(out, 2))
-    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: act, qweight must be 16-byte and scales, zeros 8-byte aligned");
-  const int spg = (int)(group / 32);
-  const int M = (int)m, K = (int)k, N = (int)n;
-  // Words per lane: the widest load that still yields about one block per CU.
-  int w = 4;
-  if (N / 64 < 192) w = 2;
-  if (N / 32 < 192) w = 1;
-  int nw = 16;
-  // XMK_INT4_TILE="<words per lane>,<waves per block>" overrides the choice (tuning aid).
-  static const char* tile_env = getenv("XMK_INT4_TILE");
-  if (tile_env) {
-    int ew = 0, enw = 0;
-    if (sscanf(tile_env, "%d,%d", &ew, &enw) == 2 && (ew == 1 || ew == 2 || ew == 4) && (enw == 8 || enw == 16)) {
-      w = ew;
-      nw = enw;
-    }
-  }
-  SplitArgs sk;
-  if (split.ksplit > 1) {
-    if (M > 16 || !split.partial || split.ksplit > kInt4MaxSplit ||
-        split.partial_bytes < (size_t)split.ksplit * 32 * N * sizeof(float))
-      return xmk::fail(XMK_INTERNAL, "int4_gemm: bad K split request");
-    w = 4;
-    nw = 8;
-    sk.ksplit = split.ksplit;
-    sk.partial = split.partial;
-  }
-  xmk::trace("int4_gemm m=%d k=%d n=%d group=%d words_per_lane=%d waves=%d ksplit=%d", M, K, N, (int)group, w, nw,
-             sk.ksplit);
-  for (int m_base = 0; m_base < M; m_base += 32) {
-    const int rows = M - m_base;
-    int rc;
-#define XMK_INT4_ARGS spg, act, qweight, scales, zeros, bias, out, m_base, M, K, N, ep, st, sk
-#define XMK_INT4_CASE(WW)                                                   \
-  do {                                                                      \
-    if (rows > 16) rc = launch_spg<WW, 2, 4, 8>(XMK_INT4_ARGS);             \
-    else if (rows > 1) rc = launch_spg<WW, 1, 4, 8>(XMK_INT4_ARGS);         \
-    else rc = nw == 16 ? launch_spg<WW, 1, 1, 16>(XMK_INT4_ARGS)            \
-                       : launch_spg<WW, 1, 1, 8>(XMK_INT4_ARGS);            \
-  } while (0)
-    if (w == 4) XMK_INT4_CASE(4);
-    else if (w == 2) XMK_INT4_CASE(2);
-    else XMK_INT4_CASE(1);
-#undef XMK_INT4_CASE
-#undef XMK_INT4_ARGS
-    if (rc != XMK_OK) return rc;
-  }
-  return xmk::check_launch("int4_gemm");
+  Int4Call c;
+  c.act = act; c.qweight = qweight; c.scales = scales; c.zeros = zeros; c.bias = bias; c.out = out;
+  c.k = k; c.n = n; c.ep = ep; c.split = split;
+  return int4_gemm_launch2(c, nullptr, m, group, st);
 }
 
 extern "C" int xmk_int4_gemm(const void* act, const void* qweight, const void* scales,
