@@ -114,6 +114,16 @@ const char* xmk_last_error(void);
  * tiled kernel, where the reference falls back to oneDNN. */
 int xmk_gemm(const xmk_gemm_desc* desc, void* stream);
 
+/* xmk_gemm with caller-provided scratch (the reference's handlers receive a scratch allocator for
+ * this purpose, sycl_custom_call.cc:155).  When the output has too few tiles to fill the device and K
+ * is long (small-M decode shapes such as the 1_4096_4096 and 4_4096_16384 entries of the reference's
+ * table, xetla/gemm/gemm.cc:32-37, which it runs with SLM_KS k-slicing), K is split over work-groups:
+ * fp32 partial sums go to the workspace and a second kernel adds them in slice order and applies the
+ * epilogue.  xmk_gemm_workspace_bytes returns the bytes that makes possible for this descriptor
+ * (0: the call would not split).  With a NULL or too small workspace the call is xmk_gemm. */
+size_t xmk_gemm_workspace_bytes(const xmk_gemm_desc* desc);
+int xmk_gemm_ws(const xmk_gemm_desc* desc, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Three GEMMs that share the left operand: out_i = act(lhs · rhs_i + bias_i), i = q, k, v.
  * Replaces XetlaQKVGemmKernel (xetla/gemm/gemm.h:112-170) and hgemm_qkv / hgemm_qkv_bias
  * (xetla/gemm/hgemm_impl.h:461-608), which the reference launches as one kernel over a

@@ -66,7 +66,8 @@ def lib():
                               ("xmk_last_error", ctypes.c_char_p),
                               ("xmk_gemm_policy_name", ctypes.c_char_p),
                               ("xmk_fmha_decode_workspace_bytes", ctypes.c_size_t),
-                              ("xmk_fmha_bwd_workspace_bytes", ctypes.c_size_t)):
+                              ("xmk_fmha_bwd_workspace_bytes", ctypes.c_size_t),
+                              ("xmk_gemm_workspace_bytes", ctypes.c_size_t)):
             if hasattr(L, name):
                 getattr(L, name).restype = restype
         _lib = L
@@ -109,7 +110,7 @@ def run_gemm_desc(desc, stream=None):
 
 
 def run_gemm(lhs, rhs, out, *, lhs_transpose=False, rhs_transpose=False, out_transpose=False,
-             c=None, bias=None, alpha=1.0, beta=0.0, epilogue=EPI_DEFAULT, stream=None):
+             c=None, bias=None, alpha=1.0, beta=0.0, epilogue=EPI_DEFAULT, stream=None, workspace=None):
     """out = act(alpha * op(lhs) op(rhs) + beta * c + bias).  Tensors are the *stored*
     row-major matrices; ``*_transpose`` marks the operand as the transpose of what is
     stored (a column-major XLA layout)."""
@@ -118,8 +119,18 @@ def run_gemm(lhs, rhs, out, *, lhs_transpose=False, rhs_transpose=False, out_tra
                  matrix(out, out_transpose), None if c is None else c.data_ptr(),
                  None if bias is None else bias.data_ptr(), dtype_code(lhs), dtype_code(out),
                  batch, alpha, beta, epilogue)
-    run_gemm_desc(d, stream)
+    if workspace is not None:
+        _check(lib().xmk_gemm_ws(ctypes.byref(d), _ptr(workspace), ctypes.c_size_t(workspace.numel() * workspace.element_size()),
+                                 _stream(stream)))
+    else:
+        run_gemm_desc(d, stream)
     return out
+
+
+def gemm_workspace_bytes(lhs, rhs, out, *, lhs_transpose=False, rhs_transpose=False, out_transpose=False):
+    d = GemmDesc(matrix(lhs, lhs_transpose), matrix(rhs, rhs_transpose), matrix(out, out_transpose), None, None,
+                 dtype_code(lhs), dtype_code(out), 1, 1.0, 0.0, EPI_DEFAULT)
+    return lib().xmk_gemm_workspace_bytes(ctypes.byref(d))
 
 
 def run_gemm_qkv(lhs, weights, out_q, out_k, out_v, *, rhs_transpose=False, bias=None, epilogue=EPI_DEFAULT,

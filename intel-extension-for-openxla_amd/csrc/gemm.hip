@@ -128,6 +128,41 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(GenericParams p) {
   }
 }
 
+// Second pass of a K-split GEMM: out = act(alpha * sum_z partial[z] + beta * c + bias), one rounding.
+// partial: fp32 [ks][M][N] packed; out / c: [M][ldc] of kind kout; bias of kind kin.
+struct ReduceParams {
+  const float* partial;
+  void* out;
+  const void* c;
+  const void* bias;
+  int M, N, ks;
+  int64_t ldc;
+  int kin, kout;
+  float alpha, beta;
+  int act;
+};
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(ReduceParams p) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;  // four consecutive columns; N % 4 == 0
+  const int64_t total = (int64_t)p.M * p.N;
+  if (idx >= total) return;
+  const int m = (int)(idx / p.N), n = (int)(idx % p.N);
+  floatx4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int z = 0; z < p.ks; ++z) s += *reinterpret_cast<const floatx4*>(p.partial + (int64_t)z * total + idx);
+  const int64_t off = (int64_t)m * p.ldc + n;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float v = p.alpha * s[j];
+    if (p.beta != 0.f && p.c) v += p.beta * load_as_f32(p.c, p.kout, off + j);
+    if (p.bias) v += load_as_f32(p.bias, p.kin, n + j);
+    v = apply_act(v, p.act);
+    switch (p.kout) {
+      case G_BF16: reinterpret_cast<__bf16*>(p.out)[off + j] = (__bf16)v; break;
+      case G_F16: reinterpret_cast<_Float16*>(p.out)[off + j] = (_Float16)v; break;
+      default: reinterpret_cast<float*>(p.out)[off + j] = v; break;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ host side
 
 int generic_kind(int dtype) {
@@ -163,9 +198,90 @@ extern "C" const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int
 namespace {
 // out1 / out2: further outputs of the shared-lhs three-GEMM form, or null for a plain GEMM.
 int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream);
+
+// K slices worth using for a plain 16-bit GEMM of this shape when scratch is available: few
+// output tiles (the device has 256 CUs) and a long reduction.  1: do not split.
+int plan_splitk(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k) {
+  if (d->batch_size != 1 || n % 4 != 0) return 1;
+  if (d->dtype_in != XMK_BF16 && d->dtype_in != XMK_F16) return 1;
+  const Policy& pol = kPolicies[select_policy(m, n, k)];
+  const int64_t tiles = xmk::ceil_div(m, pol.bm) * xmk::ceil_div(n, pol.bn);
+  int ks = 1;
+  while (ks < 8 && tiles * ks * 2 <= 256 && k % (ks * 2 * 8) == 0 && k / (ks * 2) >= 512) ks *= 2;
+  return ks;
+}
+
+void gemm_dims(const xmk_gemm_desc* d, int64_t* m, int64_t* n, int64_t* k) {
+  const bool t = d->out.transpose != 0;  // C^T = B^T A^T swaps the roles
+  const xmk_matrix& lhs = t ? d->rhs : d->lhs;
+  const xmk_matrix& rhs = t ? d->lhs : d->rhs;
+  const bool lt = t ? !lhs.transpose : lhs.transpose, rt = t ? !rhs.transpose : rhs.transpose;
+  *m = lt ? lhs.num_cols : lhs.num_rows;
+  *k = lt ? lhs.num_rows : lhs.num_cols;
+  *n = rt ? rhs.num_rows : rhs.num_cols;
+}
 }  // namespace
 
 extern "C" int xmk_gemm(const xmk_gemm_desc* d, void* stream) { return run_gemm(d, nullptr, nullptr, stream); }
+
+extern "C" size_t xmk_gemm_workspace_bytes(const xmk_gemm_desc* d) {
+  if (!d || d->out.transpose) return 0;
+  int64_t m, n, k;
+  gemm_dims(d, &m, &n, &k);
+  if (m <= 0 || n <= 0 || k <= 0) return 0;
+  const int ks = plan_splitk(d, m, n, k);
+  return ks > 1 ? (size_t)ks * m * n * sizeof(float) : 0;
+}
+
+extern "C" int xmk_gemm_ws(const xmk_gemm_desc* d, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!d) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: null descriptor");
+  const size_t need = xmk_gemm_workspace_bytes(d);
+  if (need == 0 || !workspace || workspace_bytes < need || !xmk::aligned(workspace, 16) || d->lhs.transpose)
+    return run_gemm(d, nullptr, nullptr, stream);
+  int64_t m, n, k;
+  gemm_dims(d, &m, &n, &k);
+  const int ks = plan_splitk(d, m, n, k);
+  // Pass 1: the K slices as a batched GEMM into fp32 partial sums (no epilogue); a slice is a
+  // column range of lhs and a row (or column) range of rhs, so only the batch strides change.
+  xmk_gemm_desc p = *d;
+  const int64_t kz = k / ks;
+  p.lhs.num_cols = kz;
+  p.lhs.batch_stride = kz;
+  if (p.rhs.transpose) { p.rhs.num_cols = kz; p.rhs.batch_stride = kz; }
+  else { p.rhs.num_rows = kz; p.rhs.batch_stride = kz * p.rhs.leading_dim_stride; }
+  p.out.data = workspace; p.out.leading_dim_stride = n; p.out.batch_stride = m * n;
+  p.c = nullptr; p.bias = nullptr;
+  p.dtype_out = XMK_F32;
+  p.batch_size = ks; p.alpha = 1.0f; p.beta = 0.0f; p.epilogue = XMK_EPI_DEFAULT;
+  // what the full call would have rejected must still be rejected: validate it first
+  int act = ACT_NONE;
+  bool wants_bias = false;
+  switch (d->epilogue) {
+    case XMK_EPI_DEFAULT: break;
+    case XMK_EPI_RELU: act = ACT_RELU; break;
+    case XMK_EPI_GELU: act = ACT_GELU; break;
+    case XMK_EPI_BIAS: wants_bias = true; break;
+    case XMK_EPI_BIAS_RELU: wants_bias = true; act = ACT_RELU; break;
+    case XMK_EPI_BIAS_GELU: wants_bias = true; act = ACT_GELU; break;
+    default: return run_gemm(d, nullptr, nullptr, stream);  // reports the error
+  }
+  if ((wants_bias && !d->bias) || (d->beta != 0.0f && !d->c) || !d->out.data ||
+      d->out.num_rows != m || d->out.num_cols != n || d->out.leading_dim_stride < n ||
+      (d->dtype_out != d->dtype_in && d->dtype_out != XMK_F32))
+    return run_gemm(d, nullptr, nullptr, stream);  // reports the error
+  xmk::trace("gemm m=%lld n=%lld k=%lld -> split K %d ways", (long long)m, (long long)n, (long long)k, ks);
+  int rc = run_gemm(&p, nullptr, nullptr, stream);
+  if (rc != XMK_OK) return rc;
+  ReduceParams r;
+  r.partial = (const float*)workspace; r.out = d->out.data; r.c = d->beta != 0.0f ? d->c : nullptr;
+  r.bias = wants_bias ? d->bias : nullptr;
+  r.M = (int)m; r.N = (int)n; r.ks = ks; r.ldc = d->out.leading_dim_stride;
+  r.kin = generic_kind(d->dtype_in); r.kout = generic_kind(d->dtype_out);
+  r.alpha = d->alpha; r.beta = d->beta; r.act = act;
+  hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)xmk::ceil_div(m * n / 4, 256)), dim3(256), 0,
+                     (hipStream_t)stream, r);
+  return xmk::check_launch("gemm");
+}
 
 extern "C" int xmk_gemm_qkv(const xmk_gemm_desc* d, void* out_k, void* out_v, void* stream) {
   if (!d) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm_qkv: null descriptor");

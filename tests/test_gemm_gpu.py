@@ -225,3 +225,31 @@ def test_qkv_fused_gemm(xmk, oracle, dt_name, m, n, k, rhs_t, with_bias):
                  epilogue=xmk.EPI_BIAS if with_bias else xmk.EPI_DEFAULT)
     torch.cuda.synchronize()
     assert torch.equal(sep.view(torch.int16), outs[1].view(torch.int16))
+
+
+@pytest.mark.parametrize("dt_name", ["BF16", "F16"])
+@pytest.mark.parametrize("m,n,k,rhs_t,epi", [(1, 4096, 4096, False, "EPI_DEFAULT"), (4, 4096, 16384, True, "EPI_BIAS_GELU"),
+                                             (16, 1024, 8192, False, "EPI_BIAS"), (3, 520, 2048, True, "EPI_RELU")])
+def test_split_k_with_workspace(xmk, oracle, dt_name, m, n, k, rhs_t, epi):
+    """Small-M decode shapes: K split over work-groups into caller scratch, second pass applies
+    the epilogue (beta * C included)."""
+    dt = getattr(oracle, dt_name)
+    kind = _kind(dt, oracle)
+    tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+    a = oracle.from_f32(oracle.normal((m, k), 80, k ** -0.5), dt)
+    b = oracle.from_f32(oracle.normal((n, k) if rhs_t else (k, n), 81, 1.0), dt)
+    c = oracle.from_f32(oracle.normal((m, n), 82, 1.0), dt)
+    bias = oracle.from_f32(oracle.normal((n,), 83, 0.5), dt) if "BIAS" in epi else None
+    _, ref = oracle.gemm(a, b, dt, dt, rhs_t=rhs_t, c=c, bias=bias, beta=0.5, epilogue=getattr(oracle, epi))
+    da, db, dc = to_dev(a, kind), to_dev(b, kind), to_dev(c, kind)
+    nbytes = xmk.gemm_workspace_bytes(da, db, dc, rhs_transpose=rhs_t)
+    assert nbytes > 0, "these shapes are meant to split"
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device="cuda")
+    xmk.run_gemm(da, db, dc, rhs_transpose=rhs_t, c=dc, beta=0.5, bias=None if bias is None else to_dev(bias, kind),
+                 epilogue=getattr(xmk, epi), workspace=ws)
+    torch.cuda.synchronize()
+    _check(oracle, dc.float().cpu().numpy(), ref[0])
+    # a large-M shape does not ask for scratch
+    big = torch.empty((2048, 4096), dtype=tdt, device="cuda")
+    w = torch.empty((4096, 4096), dtype=tdt, device="cuda")
+    assert xmk.gemm_workspace_bytes(big, w, big) == 0
