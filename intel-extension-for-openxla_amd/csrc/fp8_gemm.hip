@@ -177,6 +177,20 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
 
   // acc[i][j][e] is out[m][n], m = m0 + wm WTM + 32 i + lane%32, n = n0 + wn WTN + 32 j + 8 (e/4) + 4 (lane/32) + e%4.
   const float scale = p.a_scale[0] * p.b_scale[0];
+  static_assert(NSTAGE * STAGE >= BM * BN * 2, "the output tile is staged in the operand stages");
+  if (m0 + BM <= p.M && n0 + BN <= p.N && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(p.out) % 16 == 0) {
+    // Tile fully inside (uniform over the work-group): round, lay out row-major in LDS and copy out
+    // in whole row segments.
+    gemm_impl::GemmParams q{};
+    q.out = p.out;
+    q.ldc = p.N;
+    q.alpha = scale;
+    q.act = gemm_impl::ACT_NONE;
+    __builtin_amdgcn_s_barrier();  // every wave has read its last fragments
+    gemm_impl::store_tile_via_lds<__bf16, false, WTM, WTN, TM, TN>(q, acc, lds + wave * (WTM * WTN * 2),
+                                                                   m0 + wm * WTM, n0 + wn * WTN, 0, lane);
+    return;
+  }
   static_for<TM>([&](auto I) {
     constexpr int i = decltype(I)::value;
     const int m = m0 + wm * WTM + i * 32 + (lane & 31);

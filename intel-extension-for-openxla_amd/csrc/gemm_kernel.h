@@ -285,6 +285,66 @@ __device__ __forceinline__ void store_quad(const GemmParams& p, floatx4 a, int m
   }
 }
 
+// The epilogue's arithmetic for four consecutive columns n..n+3 of row m that lie inside the matrix.
+// PLAIN: alpha == 1 and no addend, bias or activation.
+template <typename T, bool PLAIN>
+__device__ __forceinline__ floatx4 quad_values(const GemmParams& p, floatx4 a, int m, int n, int64_t coff) {
+  if constexpr (PLAIN) return a;
+  float v0 = p.alpha * a[0], v1 = p.alpha * a[1], v2 = p.alpha * a[2], v3 = p.alpha * a[3];
+  if (p.c) {
+    const u32x2 cw = *reinterpret_cast<const u32x2*>(reinterpret_cast<const T*>(p.c) + coff + (int64_t)m * p.ldc + n);
+    const T* cp = reinterpret_cast<const T*>(&cw);
+    v0 += p.beta * Elem<T>::to_f32(cp[0]); v1 += p.beta * Elem<T>::to_f32(cp[1]);
+    v2 += p.beta * Elem<T>::to_f32(cp[2]); v3 += p.beta * Elem<T>::to_f32(cp[3]);
+  }
+  if (p.bias) {
+    const T* bp = reinterpret_cast<const T*>(p.bias) + n;
+    v0 += Elem<T>::to_f32(bp[0]); v1 += Elem<T>::to_f32(bp[1]);
+    v2 += Elem<T>::to_f32(bp[2]); v3 += Elem<T>::to_f32(bp[3]);
+  }
+  return floatx4{apply_act(v0, p.act), apply_act(v1, p.act), apply_act(v2, p.act), apply_act(v3, p.act)};
+}
+
+// Epilogue of a tile that lies fully inside a 16-bit output matrix: each wave rounds its WTM x WTN
+// part, lays it out row-major in its own LDS region, and copies the region out with 16-byte stores
+// that cover whole row segments (the accumulator layout itself gives a lane 8 bytes in each of 32
+// different rows per store).  XOR on the 16-byte chunk index keeps both passes off the same banks.
+template <typename T, bool PLAIN, int WTM, int WTN, int TM, int TN>
+__device__ __forceinline__ void store_tile_via_lds(const GemmParams& q, const floatx16 (&acc)[TM][TN], char* region,
+                                                   int m_base, int n_base, int64_t coff, int lane) {
+  constexpr int RBY = WTN * 2;       // bytes per row of the region
+  constexpr int CPRW = RBY / 16;     // 16-byte chunks per row (4, 8 or 16)
+  constexpr int RDIV = 16 / CPRW;    // rows that share one 256-byte bank sweep
+  static_assert(CPRW == 4 || CPRW == 8 || CPRW == 16, "unsupported wave tile width");
+  const int r1 = lane & 31;
+  const int s1 = (r1 / RDIV) & (CPRW - 1);
+  static_for<TM>([&](auto I) {
+    constexpr int i = decltype(I)::value;
+    static_for<TN>([&](auto J) {
+      constexpr int j = decltype(J)::value;
+      const floatx16 t = acc[i][j];
+      static_for<4>([&](auto Q) {
+        constexpr int qd = decltype(Q)::value;
+        const floatx4 v = quad_values<T, PLAIN>(q, floatx4{t[4 * qd], t[4 * qd + 1], t[4 * qd + 2], t[4 * qd + 3]},
+                                                m_base + i * 32 + r1, n_base + j * 32 + 8 * qd + 4 * (lane >> 5), coff);
+        u32x2 w;
+        w[0] = (uint32_t)Elem<T>::from_f32(v[0]) | ((uint32_t)Elem<T>::from_f32(v[1]) << 16);
+        w[1] = (uint32_t)Elem<T>::from_f32(v[2]) | ((uint32_t)Elem<T>::from_f32(v[3]) << 16);
+        *reinterpret_cast<u32x2*>(region + (i * 32 + r1) * RBY + (((4 * j + qd) ^ s1) << 4) + (lane >> 5) * 8) = w;
+      });
+    });
+  });
+  constexpr int RPI = 64 / CPRW;  // rows per copy instruction
+  uint16_t* out = reinterpret_cast<uint16_t*>(q.out) + coff + (int64_t)m_base * q.ldc + n_base + (lane % CPRW) * 8;
+#pragma unroll 4
+  for (int it = 0; it < WTM / RPI; ++it) {
+    const int row = it * RPI + lane / CPRW;
+    const int chunk = (lane % CPRW) ^ ((row / RDIV) & (CPRW - 1));
+    const u32x4 v = *reinterpret_cast<const u32x4*>(region + row * RBY + (chunk << 4));
+    *reinterpret_cast<u32x4*>(out + (int64_t)row * q.ldc) = v;
+  }
+}
+
 // T: element type; OutF32: fp32 output (else T); A_MC / B_MC: operand's free index is
 // contiguous; BM x BN tile; WGM x WGN waves; BK: K step (32 or 64); NSTAGE: LDS stages.
 template <typename T, bool OutF32, bool A_MC, bool B_MC, int BM, int BN, int WGM, int WGN, int BK, int NSTAGE>
@@ -444,6 +504,22 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   GemmParams q = p;  // this batch member's view of the output and bias
   if (p.out_alt[0] && bz > 0) q.out = p.out_alt[bz - 1];
   if (p.bias) q.bias = reinterpret_cast<const T*>(p.bias) + bz * p.sbias;
+  if constexpr (!OutF32) {
+    static_assert(NSTAGE * STAGE >= BM * BN * 2, "the output tile is staged in the operand stages");
+    const bool inside = m0 + BM <= p.M && n0 + BN <= p.N && p.ldc % 8 == 0 &&
+                        (reinterpret_cast<uintptr_t>(q.out) + coff * 2) % 16 == 0 &&
+                        (!p.c || (p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.c) + coff * 2) % 8 == 0));
+    if (inside) {                      // uniform over the work-group
+      __builtin_amdgcn_s_barrier();    // every wave has read its last fragments
+      char* region = lds + wave * (WTM * WTN * 2);
+      const int mb = m0 + wm * WTM, nb = n0 + wn * WTN;
+      if (p.alpha == 1.0f && !p.c && !p.bias && p.act == ACT_NONE)
+        store_tile_via_lds<T, true, WTM, WTN, TM, TN>(q, acc, region, mb, nb, coff, lane);
+      else
+        store_tile_via_lds<T, false, WTM, WTN, TM, TN>(q, acc, region, mb, nb, coff, lane);
+      return;
+    }
+  }
   static_for<TM>([&](auto I) {
     constexpr int i = decltype(I)::value;
     const int m = m0 + wm * WTM + i * 32 + (lane & 31);
