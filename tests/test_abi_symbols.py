@@ -1,5 +1,5 @@
-"""The C-ABI library loads without a GPU and exports every entry point declared in include/xmk.h
-and include/xmk_ffi.h.
+"""The C-ABI library loads without a GPU and exports every entry point declared in include/xmk.h,
+include/xmk_ffi.h and include/xmk_probe.h.
 
 No compute entry point is called here; argument validation that returns before any device work
 (null descriptors, bad dtypes) is exercised because it must hold on a host without a GPU too."""
@@ -10,7 +10,7 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("xmk.h", "xmk_ffi.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("xmk.h", "xmk_ffi.h", "xmk_probe.h")]
 LIB = os.path.join(ROOT, "intel-extension-for-openxla_amd", "libxmk.so")
 
 
@@ -36,13 +36,13 @@ def test_header_declares_the_expected_surface():
                      "xmk_fmha_decode", "xmk_gptj_decode_step", "xmk_last_error", "xmk_version",
                      "xmk_ffi_cublas_gemm", "xmk_ffi_cublas_lt_matmul", "xmk_ffi_fmha_softmax",
                      "xmk_ffi_fmha_scale_bias_softmax", "xmk_ffi_int4_gemm", "xmk_ffi_cublas_lt_matmul_f8",
-                     "xmk_ffi_targets", "xmk_ffi_register_all"):
+                     "xmk_ffi_targets", "xmk_ffi_register_all", "xmk_probe_mfma_rate", "xmk_probe_mfma_flops"):
         assert required in names, names
 
 
 def test_every_declared_symbol_is_exported(lib):
     missing = [n for n in declared_entry_points() if not hasattr(lib, n)]
-    assert not missing, f"declared in xmk.h but not exported: {missing}"
+    assert not missing, f"declared in include/*.h but not exported: {missing}"
 
 
 def test_version_and_error_strings(lib):
