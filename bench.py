@@ -26,9 +26,9 @@ HBM_PEAK = 8000.0                                        # GB/s
 # profiles/hbm_traffic_pmc.txt; a workload without a measurement reports null.
 TRAFFIC_BYTES = {
     "fmha_causal": (196700 * 2.0 + 131100) * 1024,
-    "gemm_8192": (790800 * 2.0 + 132800) * 1024,
+    "gemm_8192": (791700 * 2.0 + 131100) * 1024,
     "int4_m1": (17480 * 2.0 + 32) * 1024,
-    "fp8_8192": (393400 * 2.0 + 265800) * 1024,
+    "fp8_8192": (393600 * 2.0 + 131100) * 1024,
 }
 
 
