@@ -122,7 +122,9 @@ __host__ __device__ constexpr int wait_vm_lgkm0(int n) { return (n & 0xf) | ((n 
 
 // T: element type; HP: head size padded to 64 / 128 / 256; QT: 32-row query tiles per wave;
 // NW: waves per work-group; WPS: waves per SIMD the register budget is set for.
-template <typename T, int HP, int QT, int NW, int WPS, bool CAUSAL, bool BIAS>
+// BIAS: 0 none; 1 read from global memory element by element (any shape and alignment); 2 staged
+// through LDS one [rows x 64 keys] tile per key block (T % 8 == 0, 16-byte aligned bias).
+template <typename T, int HP, int QT, int NW, int WPS, bool CAUSAL, int BIAS>
 __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   typedef typename Elem<T>::vec8 V8;
   constexpr int BR = NW * QT * 32;           // query rows per work-group
@@ -137,7 +139,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   constexpr int KS = HP / 16;                // k-steps of the S product
   constexpr int HT = HP / 32;                // 32-wide h tiles of O
   static_assert(NL >= 1 && LROWS % 8 == 0 && (2 * LROWS) % (KMASK + 1) == 0, "tile / wave split");
-  __shared__ __attribute__((aligned(1024))) char lds[4 * TILE];
+  constexpr int BTILE = 32 * BC * 2;         // one wave's bias tile: its 32 query rows x 64 keys
+  static_assert(BIAS != 2 || (QT == 1 && BC == 64), "bias staging is laid out for one 32 x 64 tile per wave");
+  __shared__ __attribute__((aligned(1024))) char lds[4 * TILE + (BIAS == 2 ? NW * BTILE : 0)];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -228,6 +232,45 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
     }
   }
 
+  // ---- bias tile (BIAS == 2): each wave keeps the [32 rows x 64 keys] tile of its own query rows in
+  // its own 4 KiB of LDS, loaded with four 1 KiB direct loads (8 rows of 128 bytes each) one block
+  // ahead.  Row r stores its 16-byte chunk c at position c ^ ((r >> 1) & 7), so that the 8-byte reads
+  // of 32 lanes (32 rows, one chunk column) spread over the banks.
+  uint32_t boff[4];  // global byte offset of this lane's chunk in load i, from bias row q0, key 0
+  int bkey[4];       // first key (within the block) of that chunk
+  int bread[8];      // LDS byte offset of the 4 keys 32 kt + 8 q + 4 g .. +3 of this lane's row: [4 kt + q]
+  const T* bias_base = nullptr;
+  if constexpr (BIAS == 2) {
+    bias_base = reinterpret_cast<const T*>(p.bias) + ((int64_t)unit * F + q0) * Tk;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 8 * i + (lane >> 3);
+      const int c = (lane & 7) ^ ((row >> 1) & 7);
+      bkey[i] = c * 8;
+      boff[i] = wq0 + row < F ? (uint32_t)((((int64_t)(wave * 32 + row)) * Tk + c * 8) * 2) : kOob;
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r) bread[r] = l32 * 128 + ((r ^ ((l32 >> 1) & 7)) << 4) + g * 8;
+  }
+  // Loads the bias tile of the key block that starts at t0.  T % 8 == 0, so a chunk lies inside
+  // the row or past its end as a whole; rows past F and chunks past T load zeros.
+  auto issue_bias = [&](int t0, char* __restrict__ btile) {
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(bias_base, 0x7fffffffu);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t off = (t0 + bkey[i] < Tk && boff[i] != kOob) ? boff[i] + (uint32_t)t0 * 2 : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(btile + i * 1024), 16, off, 0, 0, 0);
+    }
+  };
+  auto bias_value = [](u32x2 w, int e) -> float {
+    const uint32_t d = w[e >> 1];
+    if constexpr (sizeof(T) == 2 && __is_same(T, __bf16)) {
+      return __builtin_bit_cast(float, (e & 1) ? (d & 0xffff0000u) : (d << 16));
+    } else {
+      return (float)__builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? (d >> 16) : (d & 0xffffu)));
+    }
+  };
+
   floatx16 ot[QT][HT];
   float m_run[QT], l_run[QT];  // l_run: this lane's share (its 32 keys of every block) of the row sum
 #pragma unroll
@@ -259,10 +302,16 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   // Bias, masks, block max and (rarely) the rescale of tile t; returns the exponent reference.
   // st[kt][i] <-> key t0 + 32 kt + 8 (i/4) + 4 g + i%4.  Scores stay unscaled; the scale is
   // folded into the exponent.
-  auto prepare = [&](auto TI, floatx16 (&st)[2], int t0) -> float {
+  auto prepare = [&](auto TI, floatx16 (&st)[2], int t0, const u32x2 (&bv)[8]) -> float {
     constexpr int t = decltype(TI)::value;
     const int qrow = wq0 + 32 * t + l32;
-    if constexpr (BIAS) {
+    if constexpr (BIAS == 2) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) st[kt][i] += bias_value(bv[4 * kt + i / 4], i % 4) * inv_scale;
+    }
+    if constexpr (BIAS == 1) {
       if (qrow < F) {
         const T* bp = reinterpret_cast<const T*>(p.bias) + ((int64_t)unit * F + qrow) * Tk;
 #pragma unroll
@@ -349,8 +398,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   issue_tile(K, 0, kst0, koff, KV);
   if (nblk > 1) issue_tile(K, BC, kst0 + TILE, koff, KV);
   issue_tile(V, 0, vst0, &voff, 1);
-  if (nblk > 1) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(2 * NL));
-  else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(NL));
+  char* const btile0 = lds + 4 * TILE + wave * BTILE;  // this wave's bias tile (BIAS == 2)
+  constexpr int NB = BIAS == 2 ? 4 : 0;                // loads of one bias tile
+  if constexpr (BIAS == 2) issue_bias(0, btile0);
+  if (nblk > 1) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(2 * NL + NB));
+  else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(NL + NB));
   __builtin_amdgcn_s_barrier();
   floatx16 st_a[QT][2], st_b[QT][2];
   scores(kst0, st_a);
@@ -362,13 +414,24 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   // of tile 0 (VALU), the P V product of tile 0 among those of tile 1.  The four tile pointers
   // never overlap (__restrict__), so the compiler does not make the fragment reads wait for the
   // loads in flight.
+  // With a staged bias, the block first takes its bias tile out of LDS (it landed during the
+  // previous block) and then sends the next block's tile into the same 4 KiB.
   auto block = [&](int it, floatx16 (&sc)[QT][2], floatx16 (&sn)[QT][2], const char* __restrict__ knext,
-                   const char* __restrict__ vcur, char* __restrict__ kfree, char* __restrict__ vfree) {
+                   const char* __restrict__ vcur, char* __restrict__ kfree, char* __restrict__ vfree,
+                   char* __restrict__ btile) {
     const int t0 = it * BC;
+    u32x2 bv[8];
+    if constexpr (BIAS == 2) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) bv[r] = *reinterpret_cast<const u32x2*>(btile + bread[r]);
+    }
     if (it + 2 < nblk) issue_tile(K, t0 + 2 * BC, kfree, koff, KV);
     if (it + 1 < nblk) issue_tile(V, t0 + BC, vfree, &voff, 1);
+    if constexpr (BIAS == 2) {
+      if (it + 1 < nblk) issue_bias(t0 + BC, btile);
+    }
     float mref[QT];
-    static_for<QT>([&](auto TI) { mref[decltype(TI)::value] = prepare(TI, sc[decltype(TI)::value], t0); });
+    static_for<QT>([&](auto TI) { mref[decltype(TI)::value] = prepare(TI, sc[decltype(TI)::value], t0, bv); });
     V8 pf[QT][4];
     // Past the last block this reads a stale tile: finite or not, S_{nblk} is never used.
     scores(knext, sn);
@@ -406,8 +469,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
 
   for (int it = 0; it < nblk; it += 2) {
     // K_{it+1} sits in K stage 1, V_it in V stage 0; K_{it+2} goes to K stage 0, V_{it+1} to V stage 1.
-    block(it, st_a, st_b, kst0 + TILE, vst0, kst0, vst0 + TILE);
-    if (it + 1 < nblk) block(it + 1, st_b, st_a, kst0, vst0 + TILE, kst0 + TILE, vst0);
+    block(it, st_a, st_b, kst0 + TILE, vst0, kst0, vst0 + TILE, btile0);
+    if (it + 1 < nblk) block(it + 1, st_b, st_a, kst0, vst0 + TILE, kst0 + TILE, vst0, btile0);
   }
 
   // ---- finish: O = O^T / l; LSE = m ln2 + ln l.
@@ -440,22 +503,25 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
 }
 
 template <typename T, int HP, int QT, int NW, int WPS>
-void launch_cfg(FmhaParams p, uint64_t units, uint32_t F, bool causal, bool bias, hipStream_t st) {
+void launch_cfg(FmhaParams p, uint64_t units, uint32_t F, bool causal, int bias, hipStream_t st) {
   p.nqb = (int)((F + NW * QT * 32 - 1) / (NW * QT * 32));
   p.total = (int)(units * p.nqb);
   p.per_xcd = (p.total + 7) / 8;
   const dim3 grid((unsigned)(p.per_xcd * 8)), block(NW * 64);
+  // bias: 0 none, 1 element-wise from global memory, 2 staged through LDS
   if (causal) {
-    if (bias) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, true, true>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, true, false>), grid, block, 0, st, p);
+    if (bias == 2) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, true, 2>), grid, block, 0, st, p);
+    else if (bias == 1) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, true, 1>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, true, 0>), grid, block, 0, st, p);
   } else {
-    if (bias) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, false, true>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, false, false>), grid, block, 0, st, p);
+    if (bias == 2) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, false, 2>), grid, block, 0, st, p);
+    else if (bias == 1) hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, false, 1>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((fmha_fwd_kernel<T, HP, QT, NW, WPS, false, 0>), grid, block, 0, st, p);
   }
 }
 
 template <typename T>
-void launch_t(const FmhaParams& p, uint64_t units, uint32_t F, bool causal, bool bias, hipStream_t st) {
+void launch_t(const FmhaParams& p, uint64_t units, uint32_t F, bool causal, int bias, hipStream_t st) {
   // Head-size classes of the reference's policy choice (fmha_forward.h:622-646).  Two query tiles
   // per wave where the accumulators fit in the register file (head size <= 128).
   if (p.H <= 64) launch_cfg<T, 64, 1, 4, 2>(p, units, F, causal, bias, st);
@@ -495,7 +561,12 @@ extern "C" int xmk_fmha_fwd(const void* query, const void* key, const void* valu
   xmk::trace("fmha_fwd B=%u N=%u F=%u T=%u H=%u causal=%d bias=%d lse=%d", num_batches, num_heads,
              num_queries, num_keys, head_size, causal, bias != nullptr, lse != nullptr);
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == XMK_BF16) launch_t<__bf16>(p, units, num_queries, causal != 0, bias != nullptr, st);
-  else launch_t<_Float16>(p, units, num_queries, causal != 0, bias != nullptr, st);
+  // The staged bias path needs whole 16-byte chunks per row and offsets inside one query block
+  // that fit the 31-bit buffer offset.
+  const int bias_mode = !bias ? 0
+                        : (num_keys % 8 == 0 && xmk::aligned(bias, 16) && (uint64_t)num_keys * 2 * 128 < kOob) ? 2
+                                                                                                            : 1;
+  if (dtype == XMK_BF16) launch_t<__bf16>(p, units, num_queries, causal != 0, bias_mode, st);
+  else launch_t<_Float16>(p, units, num_queries, causal != 0, bias_mode, st);
   return xmk::check_launch("fmha_fwd");
 }

@@ -88,11 +88,30 @@ def test_reference_mha_shapes(xmk, oracle, name, shape):
 
 @pytest.mark.parametrize("name", ["bf16", "fp16"])
 @pytest.mark.parametrize("causal,use_bias", [(True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("F,T,H", [(130, 200, 128), (64, 333, 64), (257, 129, 256), (1, 77, 80), (200, 64, 8)])
+@pytest.mark.parametrize("F,T,H", [(130, 200, 128), (64, 333, 64), (257, 129, 256), (1, 77, 80), (200, 64, 8),
+                                   (384, 512, 64), (100, 264, 256)])
 def test_masks_bias_lse(xmk, oracle, name, causal, use_bias, F, T, H):
     """Causal (top-left aligned, fmha_utils.h:45-96), additive bias [B,N,F,T], ragged F/T (padding
-    mask, fmha_forward.h:313-318), LSE output (fmha_forward.h:433-450)."""
+    mask, fmha_forward.h:313-318), LSE output (fmha_forward.h:433-450).  Key counts that are multiples
+    of 8 take the bias through LDS tiles, the others element by element from global memory."""
     _run(xmk, oracle, name, 2, 3, F, T, H, causal=causal, use_bias=use_bias, lse=True, seed=F * 7 + T)
+
+
+def test_bias_paths_agree(xmk):
+    """The same bias through the LDS-staged path (16-byte aligned) and, from a copy that starts 2 bytes
+    later, through the element-wise path: identical scores, so identical outputs."""
+    B, N, F, T, H = 2, 2, 160, 328, 128
+    q, k, v = (torch.randn((B, N, n, H), device="cuda").bfloat16() for n in (F, T, T))
+    bias = torch.randn((B, N, F, T), device="cuda").bfloat16()
+    shifted = torch.empty((bias.numel() + 8,), dtype=torch.bfloat16, device="cuda")
+    shifted[1:1 + bias.numel()] = bias.reshape(-1)
+    bias_unaligned = shifted[1:1 + bias.numel()].view(B, N, F, T)
+    assert bias.data_ptr() % 16 == 0 and bias_unaligned.data_ptr() % 16 != 0
+    o1, o2 = torch.empty_like(q), torch.empty_like(q)
+    xmk.fmha_forward(q, k, v, o1, bias=bias)
+    xmk.fmha_forward(q, k, v, o2, bias=bias_unaligned)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2)
 
 
 def test_key_permutation_invariance(xmk):
