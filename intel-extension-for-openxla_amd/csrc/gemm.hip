@@ -363,7 +363,11 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
                     lhs.leading_dim_stride % 8 == 0 &&
                     rhs.leading_dim_stride % 8 == 0 && lhs.batch_stride % 8 == 0 &&
                     rhs.batch_stride % 8 == 0 && lhs.num_cols % 8 == 0 && rhs.num_cols % 8 == 0;
-  if (fast) {
+  // 16-bit operands that miss those conditions still run on the matrix cores, with operands gathered
+  // element by element; the output pointers must allow the epilogue's vector stores.
+  const bool gather = !fast && sixteen && xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) &&
+                      xmk::aligned(out2, 16) && xmk::aligned(d->c, 16);
+  if (fast || gather) {
     GemmParams p;
     p.a = lhs.data; p.b = rhs.data; p.out = out.data; p.c = d->beta != 0.0f ? d->c : nullptr;
     p.bias = wants_bias ? d->bias : nullptr;
@@ -373,13 +377,34 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
     p.alpha = d->alpha; p.beta = d->beta; p.act = act;
     p.out_alt[0] = out1; p.out_alt[1] = out2; p.sbias = 0;
     if (qkv) { p.sa = 0; p.sc = 0; p.sbias = n; }
+    // Widest load of the gathering kernel per operand: the pointer, the leading dimension, the batch
+    // stride and the stored row length must all be multiples of it.
+    auto widest = [](const xmk_matrix& x) {
+      int v = 8;
+      while (v > 1 && (!xmk::aligned(x.data, 2 * v) || x.leading_dim_stride % v || x.batch_stride % v || x.num_cols % v))
+        v /= 2;
+      return v;
+    };
+    p.vec_a = widest(lhs);
+    p.vec_b = widest(rhs);
     const bool a_mc = lhs.transpose != 0;   // stored [K, M]
     const bool b_mc = rhs.transpose == 0;   // stored [K, N]
-    const int pol = select_policy(m, n, k);
-    xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s",
-               (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
-               rhs.transpose, d->epilogue, d->beta, kPolicies[pol].name);
     const int batch = qkv ? 3 : (int)d->batch_size;
+    int pol = select_policy(m, n, k, batch);
+    if (gather && pol > 1) pol = 1;  // the gathering kernel exists for the two larger tiles
+    xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s%s",
+               (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
+               rhs.transpose, d->epilogue, d->beta, kPolicies[pol].name, gather ? " (gathered operands)" : "");
+    if (gather) {
+      if (din == XMK_BF16) {
+        if (dout == XMK_F32) launch_layout_gather<__bf16, true>(a_mc, b_mc, pol, p, batch, st);
+        else launch_layout_gather<__bf16, false>(a_mc, b_mc, pol, p, batch, st);
+      } else {
+        if (dout == XMK_F32) launch_layout_gather<_Float16, true>(a_mc, b_mc, pol, p, batch, st);
+        else launch_layout_gather<_Float16, false>(a_mc, b_mc, pol, p, batch, st);
+      }
+      return xmk::check_launch("gemm");
+    }
     if (din == XMK_BF16) {
       if (dout == XMK_F32) launch_layout<__bf16, true>(a_mc, b_mc, pol, p, batch, st);
       else launch_layout<__bf16, false>(a_mc, b_mc, pol, p, batch, st);

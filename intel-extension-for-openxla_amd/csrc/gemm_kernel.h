@@ -38,6 +38,9 @@ struct GemmParams {
   // out_alt[z - 1] instead of out + z * sc and reads bias + z * sbias.  Null when unused.
   void* out_alt[2];
   int64_t sbias;
+  // Gathering kernel only: elements per load (1, 2, 4 or 8) that the alignment of each operand's
+  // pointer, leading dimension, batch stride and row length allows.
+  int vec_a, vec_b;
 };
 
 __device__ __forceinline__ float gelu_tanh(float x) {
@@ -164,6 +167,50 @@ struct Loader {
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(base);
 #pragma unroll
     for (int i = 0; i < NL; ++i) issue_one(i, rsrc, kleft, lds_tile, wave);
+  }
+  // The same placement for operands the direct loads cannot take (rows that do not start on a
+  // 16-byte boundary, a row length that is not a multiple of 8): load i's chunk is gathered element
+  // by element, zero where the row, column or k does not exist, and written with one 16-byte LDS
+  // store.  Nothing outside the matrix is read.  base: tile origin for this K step; valid: rows
+  // (KC) or columns (MC) of the tile that exist; kleft as in issue_one; vec: elements per load
+  // (wave-uniform; every group of `vec` elements is aligned and lies inside the row or outside as a whole).
+  __device__ __forceinline__ void gather_one(int i, const uint16_t* base, int64_t ld, int valid, int kleft,
+                                             char* lds_tile, int wave, int lane, int vec) const {
+    scatter_one(i, gather_load(i, base, ld, valid, kleft, wave, lane, vec), lds_tile, wave, lane);
+  }
+  __device__ __forceinline__ void scatter_one(int i, u32x4 v, char* lds_tile, int wave, int lane) const {
+    *reinterpret_cast<u32x4*>(lds_tile + (i * NWAVES + wave) * 1024 + lane * 16) = v;
+  }
+  __device__ __forceinline__ u32x4 gather_load(int i, const uint16_t* base, int64_t ld, int valid, int kleft,
+                                               int wave, int lane, int vec) const {
+    const int lrow = wave * RPL + lane / CPR + i * LSTRIDE;                       // LSTRIDE % 8 == 0:
+    const int c0 = ((lane % CPR) ^ swz<MC, ROWS, BK>(wave * RPL + lane / CPR)) * 8;  // same swizzle for every i
+    const int row = MC ? c0 : lrow;   // operand row / column of element 0
+    const int k = MC ? lrow : c0;     // k (inside the K step) of element 0
+    const uint16_t* src = MC ? base + (int64_t)k * ld + row : base + (int64_t)row * ld + k;
+    const bool line = MC ? k < kleft : row < valid;  // the stored row this chunk lies in exists
+    const int left = MC ? valid - row : kleft - k;    // elements of that row from element 0 on
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (vec == 8) {
+      if (line && left > 0) v = *reinterpret_cast<const u32x4*>(src);
+    } else if (vec == 4) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (line && 4 * j < left) {
+          const u32x2 w = *reinterpret_cast<const u32x2*>(src + 4 * j);
+          v[2 * j] = w[0];
+          v[2 * j + 1] = w[1];
+        }
+    } else if (vec == 2) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (line && 2 * j < left) v[j] = *reinterpret_cast<const uint32_t*>(src + 2 * j);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (line && j < left) v[j >> 1] |= (uint32_t)src[j] << (16 * (j & 1));
+    }
+    return v;
   }
 };
 
@@ -309,9 +356,11 @@ __device__ __forceinline__ floatx4 quad_values(const GemmParams& p, floatx4 a, i
 // part, lays it out row-major in its own LDS region, and copies the region out with 16-byte stores
 // that cover whole row segments (the accumulator layout itself gives a lane 8 bytes in each of 32
 // different rows per store).  XOR on the 16-byte chunk index keeps both passes off the same banks.
+// vec: elements per global store (8, 4, 2 or 1) that the output's alignment allows; a lane always
+// owns 8 consecutive elements of a row.
 template <typename T, bool PLAIN, int WTM, int WTN, int TM, int TN>
 __device__ __forceinline__ void store_tile_via_lds(const GemmParams& q, const floatx16 (&acc)[TM][TN], char* region,
-                                                   int m_base, int n_base, int64_t coff, int lane) {
+                                                   int m_base, int n_base, int64_t coff, int lane, int vec = 8) {
   constexpr int RBY = WTN * 2;       // bytes per row of the region
   constexpr int CPRW = RBY / 16;     // 16-byte chunks per row (4, 8 or 16)
   constexpr int RDIV = 16 / CPRW;    // rows that share one 256-byte bank sweep
@@ -341,13 +390,28 @@ __device__ __forceinline__ void store_tile_via_lds(const GemmParams& q, const fl
     const int row = it * RPI + lane / CPRW;
     const int chunk = (lane % CPRW) ^ ((row / RDIV) & (CPRW - 1));
     const u32x4 v = *reinterpret_cast<const u32x4*>(region + row * RBY + (chunk << 4));
-    *reinterpret_cast<u32x4*>(out + (int64_t)row * q.ldc) = v;
+    uint16_t* dst = out + (int64_t)row * q.ldc;
+    if (vec == 8) {
+      *reinterpret_cast<u32x4*>(dst) = v;
+    } else if (vec == 4) {
+      *reinterpret_cast<u32x2*>(dst) = u32x2{v[0], v[1]};
+      *reinterpret_cast<u32x2*>(dst + 4) = u32x2{v[2], v[3]};
+    } else if (vec == 2) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *reinterpret_cast<uint32_t*>(dst + 2 * j) = v[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dst[j] = (uint16_t)(v[j >> 1] >> (16 * (j & 1)));
+    }
   }
 }
 
 // T: element type; OutF32: fp32 output (else T); A_MC / B_MC: operand's free index is
 // contiguous; BM x BN tile; WGM x WGN waves; BK: K step (32 or 64); NSTAGE: LDS stages.
-template <typename T, bool OutF32, bool A_MC, bool B_MC, int BM, int BN, int WGM, int WGN, int BK, int NSTAGE>
+// SLOW: operands are gathered element by element (Loader::gather_one) instead of loaded directly
+// into LDS; for leading dimensions and row lengths the direct loads cannot take.
+template <typename T, bool OutF32, bool A_MC, bool B_MC, int BM, int BN, int WGM, int WGN, int BK, int NSTAGE,
+          bool SLOW = false>
 __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p) {
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -405,12 +469,24 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   // vmcnt arithmetic below is uniform.
 #pragma unroll
   for (int st = 0; st < NSTAGE - 1; ++st) {
-    la.issue(a_tile, p.K - st * BK, lds + st * STAGE, wave);
-    lb.issue(b_tile, p.K - st * BK, lds + st * STAGE + A_BYTES, wave);
+    if constexpr (SLOW) {
+#pragma unroll
+      for (int i = 0; i < LoaderA::NL; ++i)
+        la.gather_one(i, reinterpret_cast<const uint16_t*>(a_tile), p.lda, p.M - m0, p.K - st * BK,
+                      lds + st * STAGE, wave, lane, p.vec_a);
+#pragma unroll
+      for (int i = 0; i < LoaderB::NL; ++i)
+        lb.gather_one(i, reinterpret_cast<const uint16_t*>(b_tile), p.ldb, p.N - n0, p.K - st * BK,
+                      lds + st * STAGE + A_BYTES, wave, lane, p.vec_b);
+    } else {
+      la.issue(a_tile, p.K - st * BK, lds + st * STAGE, wave);
+      lb.issue(b_tile, p.K - st * BK, lds + st * STAGE + A_BYTES, wave);
+    }
     a_tile += a_step;
     b_tile += b_step;
   }
-  __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 2) * LOADS));  // step 0 has landed (loads return in order)
+  if constexpr (SLOW) __builtin_amdgcn_s_waitcnt(0xc07f);                   // the gathers' LDS stores are done
+  else __builtin_amdgcn_s_waitcnt(vmcnt_imm((NSTAGE - 2) * LOADS));         // step 0 has landed (loads return in order)
   __builtin_amdgcn_s_barrier();
 
   FragAddr<A_MC, BM, BK, TM> faddr;
@@ -458,6 +534,17 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
     constexpr bool CHECK_K = decltype(CHECK)::value;
     const int kleft = p.K - (kt + NSTAGE - 1) * BK;
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(a_tile), rb = make_rsrc(b_tile);
+    // Gathering kernel: the whole K step's operand chunks are loaded into registers up front and go
+    // to LDS after the step's MFMAs, which cover most of the load latency.
+    u32x4 ga[SLOW ? LoaderA::NL : 1], gb[SLOW ? LoaderB::NL : 1];
+    if constexpr (SLOW) {
+#pragma unroll
+      for (int i = 0; i < LoaderA::NL; ++i)
+        ga[i] = la.gather_load(i, reinterpret_cast<const uint16_t*>(a_tile), p.lda, p.M - m0, kleft, wave, lane, p.vec_a);
+#pragma unroll
+      for (int i = 0; i < LoaderB::NL; ++i)
+        gb[i] = lb.gather_load(i, reinterpret_cast<const uint16_t*>(b_tile), p.ldb, p.N - n0, kleft, wave, lane, p.vec_b);
+    }
     static_for<KS>([&](auto KSI) {
       constexpr int ks = decltype(KSI)::value;
       // this k-step's share of the loads
@@ -468,15 +555,24 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
                                    ~(0xf << 8));  // and lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
       }
+      if constexpr (!SLOW) {
 #pragma unroll
-      for (int i = la0; i < la1; ++i) la.template issue_one<CHECK_K>(i, ra, kleft, wr, wave);
+        for (int i = la0; i < la1; ++i) la.template issue_one<CHECK_K>(i, ra, kleft, wr, wave);
 #pragma unroll
-      for (int i = lb0; i < lb1; ++i) lb.template issue_one<CHECK_K>(i, rb, kleft, wr + A_BYTES, wave);
+        for (int i = lb0; i < lb1; ++i) lb.template issue_one<CHECK_K>(i, rb, kleft, wr + A_BYTES, wave);
+      }
       if constexpr (ks + 1 < KS) read_frags(cur, ks + 1, (ks + 1) & 1);
       else read_frags(nxt, 0, KS & 1);
       mma(ks & 1);
-      interleave((la1 - la0) + (lb1 - lb0));
+      interleave(SLOW ? 0 : (la1 - la0) + (lb1 - lb0));
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (SLOW && ks + 1 == KS) {
+#pragma unroll
+        for (int i = 0; i < LoaderA::NL; ++i) la.scatter_one(i, ga[i], wr, wave, lane);
+#pragma unroll
+        for (int i = 0; i < LoaderB::NL; ++i) lb.scatter_one(i, gb[i], wr + A_BYTES, wave, lane);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     });
     a_tile += a_step;
     b_tile += b_step;
@@ -506,17 +602,19 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
   if (p.bias) q.bias = reinterpret_cast<const T*>(p.bias) + bz * p.sbias;
   if constexpr (!OutF32) {
     static_assert(NSTAGE * STAGE >= BM * BN * 2, "the output tile is staged in the operand stages");
-    const bool inside = m0 + BM <= p.M && n0 + BN <= p.N && p.ldc % 8 == 0 &&
-                        (reinterpret_cast<uintptr_t>(q.out) + coff * 2) % 16 == 0 &&
+    const bool inside = m0 + BM <= p.M && n0 + BN <= p.N &&
                         (!p.c || (p.ldc % 4 == 0 && (reinterpret_cast<uintptr_t>(p.c) + coff * 2) % 8 == 0));
     if (inside) {                      // uniform over the work-group
       __builtin_amdgcn_s_barrier();    // every wave has read its last fragments
       char* region = lds + wave * (WTM * WTN * 2);
       const int mb = m0 + wm * WTM, nb = n0 + wn * WTN;
+      int vec = 8;  // widest store that every row start of this batch member's output allows
+      while (vec > 1 && (p.ldc % vec != 0 || (reinterpret_cast<uintptr_t>(q.out) + coff * 2) % (2 * vec) != 0))
+        vec >>= 1;
       if (p.alpha == 1.0f && !p.c && !p.bias && p.act == ACT_NONE)
-        store_tile_via_lds<T, true, WTM, WTN, TM, TN>(q, acc, region, mb, nb, coff, lane);
+        store_tile_via_lds<T, true, WTM, WTN, TM, TN>(q, acc, region, mb, nb, coff, lane, vec);
       else
-        store_tile_via_lds<T, false, WTM, WTN, TM, TN>(q, acc, region, mb, nb, coff, lane);
+        store_tile_via_lds<T, false, WTM, WTN, TM, TN>(q, acc, region, mb, nb, coff, lane, vec);
       return;
     }
   }
@@ -557,15 +655,16 @@ struct TunedShape {
   int m, n, k, policy;
 };
 #include "gemm_policy_table.h"
-inline int select_policy(int64_t m, int64_t n, int64_t k) {
+inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1) {
   static const int forced = [] {
     const char* e = getenv("XMK_GEMM_POLICY");
     const int v = e ? atoi(e) : -1;
     return (e && v >= 0 && v < kNumPolicies) ? v : -1;
   }();
   if (forced >= 0) return forced;
-  for (const TunedShape& t : kTunedShapes)
-    if (t.m == m && t.n == n && t.k == k) return t.policy;
+  if (batch == 1)
+    for (const TunedShape& t : kTunedShapes)
+      if (t.m == m && t.n == n && t.k == k) return t.policy;
   // Heuristic: the policy with the best estimated throughput = (what the tile sustains when the
   // device is full) x (share of the 256 CUs busy over the tile waves) x (share of the tiles' area
   // inside the matrix).  The per-tile figures are measured large-shape rates relative to 256x256.
@@ -573,7 +672,7 @@ inline int select_policy(int64_t m, int64_t n, int64_t k) {
   int best = kNumPolicies - 1;
   float best_score = -1.0f;
   for (int i = 0; i < kNumPolicies; ++i) {
-    const int64_t tiles = xmk::ceil_div(m, kPolicies[i].bm) * xmk::ceil_div(n, kPolicies[i].bn);
+    const int64_t tiles = xmk::ceil_div(m, kPolicies[i].bm) * xmk::ceil_div(n, kPolicies[i].bn) * batch;
     const int64_t waves = xmk::ceil_div(tiles, 256);
     const float busy = (float)tiles / (float)(waves * 256);
     const float inside = (float)((double)m * (double)n / ((double)tiles * kPolicies[i].bm * kPolicies[i].bn));
@@ -586,9 +685,10 @@ inline int select_policy(int64_t m, int64_t n, int64_t k) {
   return best;
 }
 
-template <typename T, bool OutF32, bool A_MC, bool B_MC, int BM, int BN, int WGM, int WGN, int BK, int NSTAGE>
+template <typename T, bool OutF32, bool A_MC, bool B_MC, int BM, int BN, int WGM, int WGN, int BK, int NSTAGE,
+          bool SLOW = false>
 void launch_mfma(const GemmParams& p, int batch, hipStream_t st) {
-  hipLaunchKernelGGL((gemm_mfma_kernel<T, OutF32, A_MC, B_MC, BM, BN, WGM, WGN, BK, NSTAGE>),
+  hipLaunchKernelGGL((gemm_mfma_kernel<T, OutF32, A_MC, B_MC, BM, BN, WGM, WGN, BK, NSTAGE, SLOW>),
                      dim3(p.tiles_m * p.tiles_n, 1, batch), dim3(WGM * WGN * 64), 0, st, p);
 }
 
@@ -613,8 +713,27 @@ void launch_layout_impl(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch,
 }
 
 
+// The gathering variant (operands the direct loads cannot take): policy 0 or 1 only.
+template <typename T, bool OutF32, bool A_MC, bool B_MC>
+void launch_policy_gather(int pol, GemmParams& p, int batch, hipStream_t st) {
+  p.tiles_m = (int)xmk::ceil_div(p.M, kPolicies[pol].bm);
+  p.tiles_n = (int)xmk::ceil_div(p.N, kPolicies[pol].bn);
+  if (pol == 0) launch_mfma<T, OutF32, A_MC, B_MC, 256, 256, 2, 2, 32, 4, true>(p, batch, st);
+  else launch_mfma<T, OutF32, A_MC, B_MC, 128, 128, 2, 2, 64, 3, true>(p, batch, st);
+}
+
+template <typename T, bool OutF32>
+void launch_layout_gather_impl(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch, hipStream_t st) {
+  if (!a_mc && !b_mc) launch_policy_gather<T, OutF32, false, false>(pol, p, batch, st);
+  else if (!a_mc && b_mc) launch_policy_gather<T, OutF32, false, true>(pol, p, batch, st);
+  else if (a_mc && !b_mc) launch_policy_gather<T, OutF32, true, false>(pol, p, batch, st);
+  else launch_policy_gather<T, OutF32, true, true>(pol, p, batch, st);
+}
+
 // Explicitly instantiated in gemm_inst_*.hip.
 template <typename T, bool OutF32>
 void launch_layout(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch, hipStream_t st);
+template <typename T, bool OutF32>
+void launch_layout_gather(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch, hipStream_t st);
 
 }  // namespace gemm_impl

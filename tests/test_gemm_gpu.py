@@ -268,3 +268,51 @@ def test_mfma_probe_runs_and_validates_arguments(xmk):
         xmk.probe_mfma_rate(sink[:1024], tile=32, iters=1)
     with pytest.raises(RuntimeError):
         xmk.probe_mfma_rate(sink, tile=8, iters=1)
+
+
+@pytest.mark.parametrize("dt_name", ["BF16", "F16"])
+@pytest.mark.parametrize("lhs_t,rhs_t,out_t", [(0, 0, 0), (0, 1, 0), (1, 0, 0), (1, 1, 0), (0, 1, 1)])
+@pytest.mark.parametrize("m,n,k", [(37, 50, 45), (300, 515, 1027), (130, 258, 77), (513, 100, 264)])
+def test_gathered_operands(xmk, oracle, dt_name, lhs_t, rhs_t, out_t, m, n, k):
+    """16-bit shapes whose rows do not start on 16-byte boundaries or whose K is not a multiple of 8
+    run on the matrix cores with gathered operands: odd sizes in every layout, both tile sizes."""
+    dt = getattr(oracle, dt_name)
+    kind = _kind(dt, oracle)
+    a = oracle.from_f32(oracle.normal((k, m) if lhs_t else (m, k), 70, 0.3), dt)
+    b = oracle.from_f32(oracle.normal((n, k) if rhs_t else (k, n), 71, 0.3), dt)
+    bias = oracle.from_f32(oracle.normal((n,), 72), dt)
+    _, ref = oracle.gemm(a, b, dt, dt, lhs_t=lhs_t, rhs_t=rhs_t, out_t=out_t, bias=None if out_t else bias,
+                         epilogue=oracle.EPI_DEFAULT if out_t else oracle.EPI_BIAS_RELU)
+    tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+    out = torch.full((n, m) if out_t else (m, n), float("nan"), dtype=tdt, device="cuda")
+    xmk.run_gemm(to_dev(a, kind), to_dev(b, kind), out, lhs_transpose=lhs_t, rhs_transpose=rhs_t,
+                 out_transpose=out_t, bias=None if out_t else to_dev(bias, kind),
+                 epilogue=xmk.EPI_DEFAULT if out_t else xmk.EPI_BIAS_RELU)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    _check(oracle, got.T if out_t else got, ref[0])
+
+
+def test_gathered_operands_batched_f32_out(xmk, oracle):
+    """Batched product with odd sizes and fp32 output through the gathering kernel, and a padded
+    leading dimension that is not a multiple of 8."""
+    dt = oracle.F16
+    bsz, m, n, k = 3, 70, 45, 100
+    a = oracle.from_f32(oracle.normal((bsz, m, k), 80, 0.3), dt)
+    b = oracle.from_f32(oracle.normal((bsz, k, n), 81, 0.3), dt)
+    out = torch.full((bsz, m, n), float("nan"), dtype=torch.float32, device="cuda")
+    xmk.run_gemm(to_dev(a, "f16"), to_dev(b, "f16"), out)
+    torch.cuda.synchronize()
+    for i in range(bsz):
+        _, ref = oracle.gemm(a[i], b[i], dt, oracle.F32)
+        _check(oracle, out[i].cpu().numpy(), ref[0])
+    # rows of 104 stored in a buffer with leading dimension 107 (odd: rows start 2-byte aligned only)
+    ap = torch.zeros((m, 107), dtype=torch.float16, device="cuda")
+    a2 = oracle.from_f32(oracle.normal((m, 104), 82, 0.3), dt)
+    b2 = oracle.from_f32(oracle.normal((104, 48), 83, 0.3), dt)
+    ap[:, :104] = to_dev(a2, "f16")
+    o2 = torch.full((m, 48), float("nan"), dtype=torch.float16, device="cuda")
+    xmk.run_gemm(ap[:, :104], to_dev(b2, "f16"), o2)
+    torch.cuda.synchronize()
+    _, ref = oracle.gemm(a2, b2, dt, dt)
+    _check(oracle, o2.float().cpu().numpy(), ref[0])
