@@ -390,18 +390,17 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
     const bool a_mc = lhs.transpose != 0;   // stored [K, M]
     const bool b_mc = rhs.transpose == 0;   // stored [K, N]
     const int batch = qkv ? 3 : (int)d->batch_size;
-    int pol = select_policy(m, n, k, batch);
-    if (gather && pol > 1) pol = 1;  // the gathering kernel exists for the two larger tiles
-    xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s%s",
+    const int pol = select_policy(m, n, k, batch);
+    xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s",
                (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
-               rhs.transpose, d->epilogue, d->beta, kPolicies[pol].name, gather ? " (gathered operands)" : "");
+               rhs.transpose, d->epilogue, d->beta, gather ? kGatherPolicy.name : kPolicies[pol].name);
     if (gather) {
       if (din == XMK_BF16) {
-        if (dout == XMK_F32) launch_layout_gather<__bf16, true>(a_mc, b_mc, pol, p, batch, st);
-        else launch_layout_gather<__bf16, false>(a_mc, b_mc, pol, p, batch, st);
+        if (dout == XMK_F32) launch_layout_gather<__bf16, true>(a_mc, b_mc, p, batch, st);
+        else launch_layout_gather<__bf16, false>(a_mc, b_mc, p, batch, st);
       } else {
-        if (dout == XMK_F32) launch_layout_gather<_Float16, true>(a_mc, b_mc, pol, p, batch, st);
-        else launch_layout_gather<_Float16, false>(a_mc, b_mc, pol, p, batch, st);
+        if (dout == XMK_F32) launch_layout_gather<_Float16, true>(a_mc, b_mc, p, batch, st);
+        else launch_layout_gather<_Float16, false>(a_mc, b_mc, p, batch, st);
       }
       return xmk::check_launch("gemm");
     }

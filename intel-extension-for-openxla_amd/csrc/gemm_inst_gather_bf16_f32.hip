@@ -3,7 +3,7 @@
 
 namespace gemm_impl {
 template <>
-void launch_layout_gather<__bf16, true>(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch, hipStream_t st) {
-  launch_layout_gather_impl<__bf16, true>(a_mc, b_mc, pol, p, batch, st);
+void launch_layout_gather<__bf16, true>(bool a_mc, bool b_mc, GemmParams& p, int batch, hipStream_t st) {
+  launch_layout_gather_impl<__bf16, true>(a_mc, b_mc, p, batch, st);
 }
 }  // namespace gemm_impl

@@ -713,27 +713,29 @@ void launch_layout_impl(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch,
 }
 
 
-// The gathering variant (operands the direct loads cannot take): policy 0 or 1 only.
+// The gathering variant (operands the direct loads cannot take) has one tile, 128x128x32 in 3
+// stages: its loads go through registers and are waited for inside the K step, so what hides their
+// latency is occupancy -- 48 KB of LDS and about 150 registers let three work-groups share a CU.
+constexpr Policy kGatherPolicy = {"mfma_128x128x32_w2x2_s3_gather", 128, 128, 2, 2, 32, 3};
 template <typename T, bool OutF32, bool A_MC, bool B_MC>
-void launch_policy_gather(int pol, GemmParams& p, int batch, hipStream_t st) {
-  p.tiles_m = (int)xmk::ceil_div(p.M, kPolicies[pol].bm);
-  p.tiles_n = (int)xmk::ceil_div(p.N, kPolicies[pol].bn);
-  if (pol == 0) launch_mfma<T, OutF32, A_MC, B_MC, 256, 256, 2, 2, 32, 4, true>(p, batch, st);
-  else launch_mfma<T, OutF32, A_MC, B_MC, 128, 128, 2, 2, 64, 3, true>(p, batch, st);
+void launch_policy_gather(GemmParams& p, int batch, hipStream_t st) {
+  p.tiles_m = (int)xmk::ceil_div(p.M, kGatherPolicy.bm);
+  p.tiles_n = (int)xmk::ceil_div(p.N, kGatherPolicy.bn);
+  launch_mfma<T, OutF32, A_MC, B_MC, 128, 128, 2, 2, 32, 3, true>(p, batch, st);
 }
 
 template <typename T, bool OutF32>
-void launch_layout_gather_impl(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch, hipStream_t st) {
-  if (!a_mc && !b_mc) launch_policy_gather<T, OutF32, false, false>(pol, p, batch, st);
-  else if (!a_mc && b_mc) launch_policy_gather<T, OutF32, false, true>(pol, p, batch, st);
-  else if (a_mc && !b_mc) launch_policy_gather<T, OutF32, true, false>(pol, p, batch, st);
-  else launch_policy_gather<T, OutF32, true, true>(pol, p, batch, st);
+void launch_layout_gather_impl(bool a_mc, bool b_mc, GemmParams& p, int batch, hipStream_t st) {
+  if (!a_mc && !b_mc) launch_policy_gather<T, OutF32, false, false>(p, batch, st);
+  else if (!a_mc && b_mc) launch_policy_gather<T, OutF32, false, true>(p, batch, st);
+  else if (a_mc && !b_mc) launch_policy_gather<T, OutF32, true, false>(p, batch, st);
+  else launch_policy_gather<T, OutF32, true, true>(p, batch, st);
 }
 
 // Explicitly instantiated in gemm_inst_*.hip.
 template <typename T, bool OutF32>
 void launch_layout(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch, hipStream_t st);
 template <typename T, bool OutF32>
-void launch_layout_gather(bool a_mc, bool b_mc, int pol, GemmParams& p, int batch, hipStream_t st);
+void launch_layout_gather(bool a_mc, bool b_mc, GemmParams& p, int batch, hipStream_t st);
 
 }  // namespace gemm_impl
