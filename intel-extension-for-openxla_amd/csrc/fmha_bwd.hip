@@ -11,7 +11,10 @@
 // also takes its scratch, dp_sum and grad_query_accum, from the caller:
 // xetla_gpu_fused_mha_runner.cc:331-339); the chunk size bounds them.  No gradient is produced
 // for the bias, as in the reference (xetla_gpu_fused_mha_runner.cc:383-385).
+#include <cstdlib>
+
 #include "common.h"
+#include "fmha_bwd_fused.h"
 
 namespace {
 
@@ -124,6 +127,16 @@ int run(const void* q, const void* k, const void* v, const void* bias, const voi
   const int64_t rows = units * F;
   hipLaunchKernelGGL(dp_sum_kernel<T>, dim3((unsigned)xmk::ceil_div(rows, 4)), dim3(256), 0, st, (const T*)o, dO,
                      dsum, rows, (int)H);
+  // Without a bias and for head sizes up to 128 the gradients come from the fused kernels, which
+  // keep the scores on chip; XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
+  {
+    static const bool composed = getenv("XMK_FMHA_BWD_COMPOSED") != nullptr;
+    const fmha_bwd_fused::Args a{q, k, v, d_o, lse, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
+    if (!bias && !composed && fmha_bwd_fused::eligible(a, (uint64_t)units)) {
+      fmha_bwd_fused::launch(a, (uint64_t)units, dtype == XMK_BF16, st);
+      return xmk::check_launch("fmha_bwd");
+    }
+  }
   const int64_t ldT = pl.ldT, sst = F * ldT;  // score buffers: row length, unit stride
   int rc;
   for (int64_t u0 = 0; u0 < units; u0 += pl.chunk) {

@@ -1,0 +1,387 @@
+// Fused multi-head attention backward for bf16 / fp16 without a score-sized intermediate
+// (the role of fmha_backward_kernel_{fp16,bf16}, xetla/sdp/sdp_backward.h:22-36).
+//
+// One kernel template, run twice with the roles of queries and keys exchanged:
+//   owner = keys    : a work-group owns 128 keys (4 waves x 32) and walks the queries in blocks of 64;
+//                     it accumulates dK = scale dS^T Q and dV = P^T dO for its keys.
+//   owner = queries : a work-group owns 128 queries and walks the keys; it accumulates dQ = scale dS K.
+// with  P = exp(scale S - LSE),  dS = P o (dP - D),  S = Q K^T,  dP = dO V^T,  D = rowsum(dO o O).
+// S and dP are recomputed in both passes (7 matrix products instead of 5) so that no gradient needs
+// atomics or a second pass over partial sums: every output element is written once, in a fixed order.
+//
+// As in the forward kernel, every product is issued so that a lane owns ONE owner row:
+//   scores  = Stream_tile . Owner^T : A operand = fragment of the streamed tile (LDS), B operand =
+//             owner fragment (registers).  The 32x32 accumulator layout puts owner row l%32 in
+//             lane l and the streamed rows in the lane's registers.
+//   acc^T  += Stream_tile^T . dS    : the accumulator registers, converted, ARE the B operand (the
+//             contraction runs over the streamed rows); the streamed tile is read with the LDS
+//             transpose loads.
+// The streamed tiles go from global memory straight into LDS, two stages.
+#include <utility>
+
+#include "common.h"
+#include "fmha_bwd_fused.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+constexpr int BS = 64;   // streamed rows per block
+constexpr int BO = 128;  // owner rows per work-group
+constexpr uint32_t kOob = 0x80000000u;
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ floatx16 mfma(vec8 a, vec8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Elem<_Float16> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ floatx16 mfma(vec8 a, vec8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ floatx16 zero16() {
+  return floatx16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+}
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff) {
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+}
+// s_waitcnt immediate (gfx9 encoding): vmcnt(n), lgkmcnt(0), expcnt untouched.
+__host__ __device__ constexpr int wait_vm_lgkm0(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4); }
+
+struct KParams {
+  const void* own1;   // owner operand of the score product:   K (owner = keys) or Q
+  const void* own2;   // owner operand of the dP product:      V (owner = keys) or dO
+  const void* strm1;  // streamed operand of the score product: Q (owner = keys) or K
+  const void* strm2;  // streamed operand of the dP product:    dO (owner = keys) or V
+  const float* lse;   // [units, F] natural-log LSE of the forward pass
+  const float* dsum;  // [units, F] D = rowsum(dO o O)
+  void* out1;         // scale * dS^T Q (dK)  or  scale * dS K (dQ)
+  void* out2;         // P^T dO (dV), owner = keys only
+  int H, F, T;
+  int nob;            // owner blocks per unit
+  int total, per_xcd;
+  float scale;
+};
+
+// T: element type; HP: head size padded to 64 or 128; OWNER_K: the work-group owns keys (else queries).
+template <typename T, int HP, bool OWNER_K, bool CAUSAL>
+__global__ __launch_bounds__(256) void fmha_bwd_kernel(KParams p) {
+  typedef typename Elem<T>::vec8 V8;
+  constexpr int NW = 4;
+  constexpr int ROWB = HP * 2;               // bytes of one tile row in LDS
+  constexpr int CPR = ROWB / 16;             // 16-byte chunks per row
+  constexpr int KMASK = CPR >= 16 ? 15 : 7;  // chunk ^= row & KMASK
+  constexpr int TILE = BS * ROWB;
+  constexpr int RPL = 1024 / ROWB;           // tile rows per 1 KiB load
+  constexpr int NL = TILE / 1024 / NW;       // loads per wave per tile
+  constexpr int LROWS = NW * RPL;            // tile rows between consecutive loads of a wave
+  constexpr int KV = (LROWS % (KMASK + 1) == 0) ? 1 : 2;  // distinct swizzles among a wave's loads
+  constexpr int KS = HP / 16;                // k-steps of the score products
+  constexpr int HT = HP / 32;                // 32-wide h tiles of the gradients
+  constexpr int STATS = 2 * BS * 4;          // LSE and D of one block's 64 query rows (owner = keys)
+  static_assert(NL >= 1 && LROWS % 8 == 0 && (2 * LROWS) % (KMASK + 1) == 0, "tile / wave split");
+  __shared__ __attribute__((aligned(1024))) char lds[4 * TILE + 2 * STATS];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g = lane >> 5, l32 = lane & 31;
+  // Each XCD (own L2) gets a contiguous range of (unit, owner block) pairs: the owner blocks of a
+  // unit stream the same tiles.
+  const int wg = (int)(blockIdx.x % 8) * p.per_xcd + (int)(blockIdx.x / 8);
+  if (wg >= p.total) return;
+  const int unit = wg / p.nob;
+  const int ob = OWNER_K ? wg % p.nob : p.nob - 1 - wg % p.nob;  // causal: heaviest blocks first
+  const int o0 = ob * BO;
+  const int H = p.H;
+  const int n_own = OWNER_K ? p.T : p.F;   // owner rows of the unit
+  const int n_str = OWNER_K ? p.F : p.T;   // streamed rows of the unit
+
+  const T* Own1 = reinterpret_cast<const T*>(p.own1) + (int64_t)unit * n_own * H;
+  const T* Own2 = reinterpret_cast<const T*>(p.own2) + (int64_t)unit * n_own * H;
+  const T* Str1 = reinterpret_cast<const T*>(p.strm1) + (int64_t)unit * n_str * H;
+  const T* Str2 = reinterpret_cast<const T*>(p.strm2) + (int64_t)unit * n_str * H;
+  const float* lse = p.lse + (int64_t)unit * p.F;
+  const float* dsum = p.dsum + (int64_t)unit * p.F;
+
+  // ---- owner fragments (B operands): this wave holds owner rows wo0 + l%32, fragment s covers
+  // h = 16 s + 8 g .. +7.
+  const int wo0 = o0 + wave * 32;
+  const int orow = wo0 + l32;
+  V8 of1[KS], of2[KS];
+  {
+    const int rows_left = n_own - o0;  // > 0
+    const __amdgpu_buffer_rsrc_t r1 = make_rsrc(Own1 + (int64_t)o0 * H, (uint32_t)rows_left * H * 2);
+    const __amdgpu_buffer_rsrc_t r2 = make_rsrc(Own2 + (int64_t)o0 * H, (uint32_t)rows_left * H * 2);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int h = 16 * s + 8 * g;
+      const uint32_t off = h < H ? (uint32_t)(((wave * 32 + l32) * H + h) * 2) : kOob;  // rows past the end are out of range
+      of1[s] = __builtin_bit_cast(V8, buf_load(r1, off));
+      of2[s] = __builtin_bit_cast(V8, buf_load(r2, off));
+    }
+  }
+  // Softmax statistics of the lane's own query row (owner = queries).
+  float own_lse2 = 0.f, own_d = 0.f;
+  if constexpr (!OWNER_K) {
+    if (orow < p.F) {
+      own_lse2 = lse[orow] * kLog2e;
+      own_d = dsum[orow];
+    }
+  }
+
+  // ---- streamed tile loads, global -> LDS, as in the forward kernel: load j = i * NW + wave fills
+  // LDS bytes [1024 j, +1024) of the tile; lane l lands at row j * RPL + l / CPR, chunk l % CPR, and
+  // fetches the global chunk that belongs there under the swizzle chunk ^= row & KMASK.
+  const int lrow = wave * RPL + lane / CPR;
+  uint32_t koff[KV];
+#pragma unroll
+  for (int v = 0; v < KV; ++v) {
+    const int row = lrow + v * LROWS;
+    const int chunk = (lane % CPR) ^ (row & KMASK);
+    koff[v] = chunk * 8 < H ? (uint32_t)((lrow * H + chunk * 8) * 2) : kOob;
+  }
+  const uint32_t lstride = (uint32_t)(LROWS * H * 2);
+  auto issue_tile = [&](const T* base, int t0, char* __restrict__ tile) {
+    const int rows_left = n_str - t0;  // > 0
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)t0 * H, 0x7fffffffu);
+    const bool full = rows_left >= BS;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const uint32_t off = (full || lrow + i * LROWS < rows_left) ? koff[i % KV] : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(tile + (i * NW + wave) * 1024), 16, off,
+                                               i * lstride, 0, 0);
+    }
+  };
+  // LSE (waves 0, 2) and D (waves 1, 3) of the block's 64 query rows, one float per lane; rows past
+  // F load zeros.  Every wave issues one load so that the load counts stay uniform.
+  auto issue_stats = [&](int t0, char* __restrict__ st) {
+    const float* src = (wave & 1) ? dsum : lse;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(src, (uint32_t)p.F * 4);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(st + (wave & 1) * (BS * 4)), 4,
+                                             (uint32_t)((t0 + lane) * 4), 0, 0, 0);
+  };
+
+  // ---- per-lane LDS offsets of the fragments
+  // Row fragment (kt, s): tile row 32 kt + l%32, logical chunk 2 s + g.
+  int kbase[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) kbase[s] = l32 * ROWB + (((2 * s + g) ^ (l32 & KMASK)) << 4);
+  // Transposed fragment (group u, h tile ht): two transpose reads; within a 16-lane block lane pl
+  // addresses tile row 16 u + 4 g + pl/4 (+8 for the second read), h = cb + 4 (pl%4) .. +3.
+  int tbase[HT][2];
+  {
+    const int pl = lane & 15;
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht) {
+      const int col = 32 * ht + ((lane >> 4) & 1) * 16 + 4 * (pl & 3);
+      const int chunk = col >> 3, within = (col & 7) * 2;
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const int row = 4 * g + (pl >> 2) + 8 * h2;  // + 16 u: does not change row & KMASK
+        tbase[ht][h2] = row * ROWB + ((chunk ^ (row & KMASK)) << 4) + within;
+      }
+    }
+  }
+
+  floatx16 acc1[HT], acc2[OWNER_K ? HT : 1];
+#pragma unroll
+  for (int i = 0; i < HT; ++i) acc1[i] = zero16();
+#pragma unroll
+  for (int i = 0; i < (OWNER_K ? HT : 1); ++i) acc2[i] = zero16();
+  const float scale2 = p.scale * kLog2e;
+
+  // Blocks of streamed rows this work-group needs.
+  //   owner = queries, causal: keys up to its last query.   owner = keys, causal: queries from its first key on.
+  const int b0 = (OWNER_K && CAUSAL) ? o0 / BS : 0;
+  const int b1 = (!OWNER_K && CAUSAL) ? (min(n_str, o0 + BO) + BS - 1) / BS : (n_str + BS - 1) / BS;
+
+  // D[streamed row][owner row] = Stream_tile . Owner^T for the 64 streamed rows of a block.
+  auto scores = [&](const char* __restrict__ tile, const V8 (&of)[KS], floatx16 (&st)[2]) {
+    st[0] = zero16();
+    st[1] = zero16();
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const u32x4 kv = *reinterpret_cast<const u32x4*>(tile + kbase[s] + kt * 32 * ROWB);
+        st[kt] = Elem<T>::mfma(__builtin_bit_cast(V8, kv), of[s], st[kt]);
+      }
+  };
+  // acc^T += Stream_tile^T . F, with F given as four B-operand fragments (group u contracts the
+  // streamed rows 16 u + {0..3, 8..11} + 4 g).
+  auto accumulate = [&](const char* __restrict__ tile, const V8 (&fr)[4], floatx16 (&acc)[HT]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int ht = 0; ht < HT; ++ht) {
+        typedef short4v __attribute__((address_space(3))) * lds_ptr;
+        const char* vt = tile + u * 16 * ROWB;
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + tbase[ht][0]));
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + tbase[ht][1]));
+        u32x4 vv;
+        vv[0] = __builtin_bit_cast(u32x2, lo)[0];
+        vv[1] = __builtin_bit_cast(u32x2, lo)[1];
+        vv[2] = __builtin_bit_cast(u32x2, hi)[0];
+        vv[3] = __builtin_bit_cast(u32x2, hi)[1];
+        acc[ht] = Elem<T>::mfma(__builtin_bit_cast(V8, vv), fr[u], acc[ht]);
+      }
+  };
+
+  char* const s1 = lds;              // streamed tiles of the score product, two stages
+  char* const s2 = lds + 2 * TILE;   // streamed tiles of the dP product, two stages
+  char* const sst = lds + 4 * TILE;  // statistics, two stages
+
+  // One block: its tiles are in `c1`, `c2`, `cst`; the next block's go to `n1`, `n2`, `nst`.
+  auto block = [&](int it, const char* __restrict__ c1, const char* __restrict__ c2, const char* __restrict__ cst,
+                   char* __restrict__ n1, char* __restrict__ n2, char* __restrict__ nst) {
+    const int t0 = it * BS;
+    if (it + 1 < b1) {
+      issue_tile(Str1, t0 + BS, n1);
+      issue_tile(Str2, t0 + BS, n2);
+      if constexpr (OWNER_K) issue_stats(t0 + BS, nst);
+    }
+    floatx16 sc[2], dp[2];
+    scores(c1, of1, sc);
+    scores(c2, of2, dp);
+    // sc[kt][i], dp[kt][i] <-> streamed row t0 + 32 kt + 8 (i/4) + 4 g + i%4, owner row `orow`.
+    V8 pf[4], df[4];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        floatx4 l2, dd;
+        if constexpr (OWNER_K) {
+          l2 = *reinterpret_cast<const floatx4*>(cst + (32 * kt + 8 * qd + 4 * g) * 4);
+          dd = *reinterpret_cast<const floatx4*>(cst + BS * 4 + (32 * kt + 8 * qd + 4 * g) * 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * qd + e;
+          const int srow = t0 + 32 * kt + 8 * qd + 4 * g + e;
+          const int q = OWNER_K ? srow : orow;
+          const int key = OWNER_K ? orow : srow;
+          const float lse2 = OWNER_K ? l2[e] * kLog2e : own_lse2;
+          const float dq = OWNER_K ? dd[e] : own_d;
+          float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, -lse2));
+          if (srow >= n_str || (CAUSAL && key > q)) pr = 0.f;
+          const float ds = pr * (dp[kt][i] - dq);
+          // fragment u = 2 kt + (qd >> 1) holds registers 8 (u & 1) .. +7 of tile kt
+          pf[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)pr;
+          df[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)ds;
+        }
+      }
+    accumulate(c1, df, acc1);
+    if constexpr (OWNER_K) accumulate(c2, pf, acc2);
+    // The next block's tiles have landed (this wave's loads; every wave's after the barrier), and
+    // this wave is done reading the tiles that the loads after the next block overwrite.
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+    __builtin_amdgcn_s_barrier();
+  };
+
+  if (b0 < b1) {
+    issue_tile(Str1, b0 * BS, s1 + (b0 & 1) * TILE);
+    issue_tile(Str2, b0 * BS, s2 + (b0 & 1) * TILE);
+    if constexpr (OWNER_K) issue_stats(b0 * BS, sst + (b0 & 1) * STATS);
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+    __builtin_amdgcn_s_barrier();
+    for (int it = b0; it < b1; ++it) {
+      if (it & 1) block(it, s1 + TILE, s2 + TILE, sst + STATS, s1, s2, sst);
+      else block(it, s1, s2, sst, s1 + TILE, s2 + TILE, sst + STATS);
+    }
+  }
+
+  // ---- store: acc^T[h][owner row] -> out[owner row][h]
+  if (orow < n_own) {
+    auto store = [&](void* out, const floatx16 (&acc)[HT], float mul) {
+      T* dst = reinterpret_cast<T*>(out) + ((int64_t)unit * n_own + orow) * H;
+      static_for<HT>([&](auto HTI) {
+        constexpr int ht = decltype(HTI)::value;
+        const floatx16 o = acc[ht];
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const int h = 32 * ht + 8 * qd + 4 * g;
+          if (h < H) {  // H % 8 == 0, so the four values are all in range
+            union { T e[4]; u32x2 w; } r;
+            r.e[0] = (T)(o[4 * qd + 0] * mul);
+            r.e[1] = (T)(o[4 * qd + 1] * mul);
+            r.e[2] = (T)(o[4 * qd + 2] * mul);
+            r.e[3] = (T)(o[4 * qd + 3] * mul);
+            *reinterpret_cast<u32x2*>(dst + h) = r.w;
+          }
+        }
+      });
+    };
+    store(p.out1, acc1, p.scale);
+    if constexpr (OWNER_K) store(p.out2, acc2, 1.0f);
+  }
+}
+
+template <typename T, int HP, bool OWNER_K>
+void launch_pass(KParams p, uint64_t units, bool causal, hipStream_t st) {
+  const int n_own = OWNER_K ? p.T : p.F;
+  p.nob = (n_own + BO - 1) / BO;
+  p.total = (int)(units * p.nob);
+  p.per_xcd = (p.total + 7) / 8;
+  const dim3 grid((unsigned)(p.per_xcd * 8)), block(256);
+  if (causal) hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, true>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, false>), grid, block, 0, st, p);
+}
+
+template <typename T, int HP>
+void launch_both(const fmha_bwd_fused::Args& a, uint64_t units, hipStream_t st) {
+  KParams p;
+  p.lse = a.lse; p.dsum = a.dsum; p.H = a.H; p.F = a.F; p.T = a.T; p.scale = a.scale;
+  p.nob = p.total = p.per_xcd = 0;
+  // owner = keys: dK, dV
+  p.own1 = a.k; p.own2 = a.v; p.strm1 = a.q; p.strm2 = a.d_o; p.out1 = a.dk; p.out2 = a.dv;
+  launch_pass<T, HP, true>(p, units, a.causal, st);
+  // owner = queries: dQ
+  p.own1 = a.q; p.own2 = a.d_o; p.strm1 = a.k; p.strm2 = a.v; p.out1 = a.dq; p.out2 = nullptr;
+  launch_pass<T, HP, false>(p, units, a.causal, st);
+}
+
+}  // namespace
+
+namespace fmha_bwd_fused {
+
+bool eligible(const Args& a, uint64_t units) {
+  return a.H <= 128 && a.H % 8 == 0 && units * ((uint64_t)((a.F > a.T ? a.F : a.T) + BO - 1) / BO) < 0x7fffffffull &&
+         (uint64_t)a.F * a.H * 2 < kOob && (uint64_t)a.T * a.H * 2 < kOob;
+}
+
+void launch(const Args& a, uint64_t units, bool bf16, hipStream_t st) {
+  if (bf16) {
+    if (a.H <= 64) launch_both<__bf16, 64>(a, units, st);
+    else launch_both<__bf16, 128>(a, units, st);
+  } else {
+    if (a.H <= 64) launch_both<_Float16, 64>(a, units, st);
+    else launch_both<_Float16, 128>(a, units, st);
+  }
+}
+
+}  // namespace fmha_bwd_fused
