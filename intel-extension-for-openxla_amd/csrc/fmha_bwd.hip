@@ -1,5 +1,6 @@
-// Fused multi-head attention backward, composed from the batched MFMA GEMM and two elementwise
-// passes over the score matrix, for a chunk of (batch, head) units at a time:
+// Multi-head attention backward: entry point, D = rowsum(dO o O), and the path for what the fused
+// kernels (fmha_bwd_fused.hip: no bias, head size <= 128) do not take -- a composition of the batched
+// MFMA GEMM and two elementwise passes over the score matrix, for a chunk of (batch, head) units at a time:
 //     D   = rowsum(dO o O)                          (dp_sum, fmha_backward.h:48)
 //     S   = Q K^T                    fp32           (GEMM)
 //     P   = exp(scale S + bias - LSE), masked       (elementwise, rounded to the operand type)

@@ -1,12 +1,12 @@
 // Fused multi-head attention backward for bf16 / fp16 without a score-sized intermediate
 // (the role of fmha_backward_kernel_{fp16,bf16}, xetla/sdp/sdp_backward.h:22-36).
 //
-// One kernel template, run twice with the roles of queries and keys exchanged:
+// One kernel template, run with the roles of queries and keys exchanged:
 //   owner = keys    : a work-group owns 128 keys (4 waves x 32) and walks the queries in blocks of 64;
-//                     it accumulates dK = scale dS^T Q and dV = P^T dO for its keys.
+//                     it accumulates dK = scale dS^T Q or dV = P^T dO for its keys (one launch each).
 //   owner = queries : a work-group owns 128 queries and walks the keys; it accumulates dQ = scale dS K.
 // with  P = exp(scale S - LSE),  dS = P o (dP - D),  S = Q K^T,  dP = dO V^T,  D = rowsum(dO o O).
-// S and dP are recomputed in both passes (7 matrix products instead of 5) so that no gradient needs
+// S (and dP) are recomputed in every pass (8 matrix products instead of 5) so that no gradient needs
 // atomics or a second pass over partial sums: every output element is written once, in a fixed order.
 //
 // As in the forward kernel, every product is issued so that a lane owns ONE owner row:
@@ -89,8 +89,14 @@ struct KParams {
 };
 
 // T: element type; HP: head size padded to 64 or 128; OWNER_K: the work-group owns keys (else queries).
-template <typename T, int HP, bool OWNER_K, bool CAUSAL>
-__global__ __launch_bounds__(256) void fmha_bwd_kernel(KParams p) {
+// DS: accumulate out1 from dS (dK or dQ); PV: accumulate out2 from P (dV, owner = keys).  The
+// keys-own work is run as two launches, one per output: with both accumulator sets and both owner
+// operands a wave needs more than half the register file, and one wave per SIMD cannot overlap its
+// matrix and vector work; recomputing S in a second launch at two waves per SIMD is faster.
+template <typename T, int HP, bool OWNER_K, bool CAUSAL, bool DS, bool PV>
+__global__ __launch_bounds__(256, 2) void fmha_bwd_kernel(KParams p) {
+  static_assert(DS || PV, "nothing to compute");
+  static_assert(!PV || OWNER_K, "P^T dO belongs to the keys-own pass");
   typedef typename Elem<T>::vec8 V8;
   constexpr int NW = 4;
   constexpr int ROWB = HP * 2;               // bytes of one tile row in LDS
@@ -142,7 +148,7 @@ __global__ __launch_bounds__(256) void fmha_bwd_kernel(KParams p) {
       const int h = 16 * s + 8 * g;
       const uint32_t off = h < H ? (uint32_t)(((wave * 32 + l32) * H + h) * 2) : kOob;  // rows past the end are out of range
       of1[s] = __builtin_bit_cast(V8, buf_load(r1, off));
-      of2[s] = __builtin_bit_cast(V8, buf_load(r2, off));
+      if constexpr (DS) of2[s] = __builtin_bit_cast(V8, buf_load(r2, off));
     }
   }
   // Softmax statistics of the lane's own query row (owner = queries).
@@ -208,11 +214,11 @@ __global__ __launch_bounds__(256) void fmha_bwd_kernel(KParams p) {
     }
   }
 
-  floatx16 acc1[HT], acc2[OWNER_K ? HT : 1];
+  floatx16 acc1[DS ? HT : 1], acc2[PV ? HT : 1];
 #pragma unroll
-  for (int i = 0; i < HT; ++i) acc1[i] = zero16();
+  for (int i = 0; i < (DS ? HT : 1); ++i) acc1[i] = zero16();
 #pragma unroll
-  for (int i = 0; i < (OWNER_K ? HT : 1); ++i) acc2[i] = zero16();
+  for (int i = 0; i < (PV ? HT : 1); ++i) acc2[i] = zero16();
   const float scale2 = p.scale * kLog2e;
 
   // Blocks of streamed rows this work-group needs.
@@ -267,36 +273,45 @@ __global__ __launch_bounds__(256) void fmha_bwd_kernel(KParams p) {
     }
     floatx16 sc[2], dp[2];
     scores(c1, of1, sc);
-    scores(c2, of2, dp);
+    if constexpr (DS) scores(c2, of2, dp);
     // sc[kt][i], dp[kt][i] <-> streamed row t0 + 32 kt + 8 (i/4) + 4 g + i%4, owner row `orow`.
     V8 pf[4], df[4];
+    // Blocks that end inside the streamed range and (causal) lie wholly on the visible side of the
+    // diagonal for every row of this wave need no mask (wave-uniform test).
+    const bool masked = t0 + BS > n_str || (CAUSAL && (OWNER_K ? wo0 + 31 > t0 : t0 + BS - 1 > wo0));
+    auto elementwise = [&](auto MASKED_T) {
+      constexpr bool MASKED = decltype(MASKED_T)::value;
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        floatx4 l2, dd;
-        if constexpr (OWNER_K) {
-          l2 = *reinterpret_cast<const floatx4*>(cst + (32 * kt + 8 * qd + 4 * g) * 4);
-          dd = *reinterpret_cast<const floatx4*>(cst + BS * 4 + (32 * kt + 8 * qd + 4 * g) * 4);
+        for (int qd = 0; qd < 4; ++qd) {
+          floatx4 l2, dd;
+          if constexpr (OWNER_K) {
+            l2 = *reinterpret_cast<const floatx4*>(cst + (32 * kt + 8 * qd + 4 * g) * 4);
+            dd = *reinterpret_cast<const floatx4*>(cst + BS * 4 + (32 * kt + 8 * qd + 4 * g) * 4);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int i = 4 * qd + e;
+            const float lse2 = OWNER_K ? l2[e] * kLog2e : own_lse2;
+            const float dq = OWNER_K ? dd[e] : own_d;
+            float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, -lse2));
+            if constexpr (MASKED) {
+              const int srow = t0 + 32 * kt + 8 * qd + 4 * g + e;
+              const int q = OWNER_K ? srow : orow;
+              const int key = OWNER_K ? orow : srow;
+              if (srow >= n_str || (CAUSAL && key > q)) pr = 0.f;
+            }
+            // fragment u = 2 kt + (qd >> 1) holds registers 8 (u & 1) .. +7 of tile kt
+            if constexpr (PV) pf[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)pr;
+            if constexpr (DS) df[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)(pr * (dp[kt][i] - dq));
+          }
         }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 4 * qd + e;
-          const int srow = t0 + 32 * kt + 8 * qd + 4 * g + e;
-          const int q = OWNER_K ? srow : orow;
-          const int key = OWNER_K ? orow : srow;
-          const float lse2 = OWNER_K ? l2[e] * kLog2e : own_lse2;
-          const float dq = OWNER_K ? dd[e] : own_d;
-          float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, -lse2));
-          if (srow >= n_str || (CAUSAL && key > q)) pr = 0.f;
-          const float ds = pr * (dp[kt][i] - dq);
-          // fragment u = 2 kt + (qd >> 1) holds registers 8 (u & 1) .. +7 of tile kt
-          pf[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)pr;
-          df[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)ds;
-        }
-      }
-    accumulate(c1, df, acc1);
-    if constexpr (OWNER_K) accumulate(c2, pf, acc2);
+    };
+    if (masked) elementwise(std::true_type{});
+    else elementwise(std::false_type{});
+    if constexpr (DS) accumulate(c1, df, acc1);
+    if constexpr (PV) accumulate(c2, pf, acc2);
     // The next block's tiles have landed (this wave's loads; every wave's after the barrier), and
     // this wave is done reading the tiles that the loads after the next block overwrite.
     __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
@@ -336,20 +351,20 @@ __global__ __launch_bounds__(256) void fmha_bwd_kernel(KParams p) {
         }
       });
     };
-    store(p.out1, acc1, p.scale);
-    if constexpr (OWNER_K) store(p.out2, acc2, 1.0f);
+    if constexpr (DS) store(p.out1, acc1, p.scale);
+    if constexpr (PV) store(p.out2, acc2, 1.0f);
   }
 }
 
-template <typename T, int HP, bool OWNER_K>
+template <typename T, int HP, bool OWNER_K, bool DS, bool PV>
 void launch_pass(KParams p, uint64_t units, bool causal, hipStream_t st) {
   const int n_own = OWNER_K ? p.T : p.F;
   p.nob = (n_own + BO - 1) / BO;
   p.total = (int)(units * p.nob);
   p.per_xcd = (p.total + 7) / 8;
   const dim3 grid((unsigned)(p.per_xcd * 8)), block(256);
-  if (causal) hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, true>), grid, block, 0, st, p);
-  else hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, false>), grid, block, 0, st, p);
+  if (causal) hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, true, DS, PV>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, false, DS, PV>), grid, block, 0, st, p);
 }
 
 template <typename T, int HP>
@@ -357,12 +372,13 @@ void launch_both(const fmha_bwd_fused::Args& a, uint64_t units, hipStream_t st) 
   KParams p;
   p.lse = a.lse; p.dsum = a.dsum; p.H = a.H; p.F = a.F; p.T = a.T; p.scale = a.scale;
   p.nob = p.total = p.per_xcd = 0;
-  // owner = keys: dK, dV
+  // owner = keys: dK, then dV
   p.own1 = a.k; p.own2 = a.v; p.strm1 = a.q; p.strm2 = a.d_o; p.out1 = a.dk; p.out2 = a.dv;
-  launch_pass<T, HP, true>(p, units, a.causal, st);
+  launch_pass<T, HP, true, true, false>(p, units, a.causal, st);
+  launch_pass<T, HP, true, false, true>(p, units, a.causal, st);
   // owner = queries: dQ
   p.own1 = a.q; p.own2 = a.d_o; p.strm1 = a.k; p.strm2 = a.v; p.out1 = a.dq; p.out2 = nullptr;
-  launch_pass<T, HP, false>(p, units, a.causal, st);
+  launch_pass<T, HP, false, true, false>(p, units, a.causal, st);
 }
 
 }  // namespace
