@@ -22,7 +22,7 @@ struct Args {
   bool causal;
 };
 
-// Head sizes up to 128 (multiples of 8), no additive bias.
+// Head sizes up to 256 (multiples of 8), no additive bias.
 bool eligible(const Args& a, uint64_t units);
 // Two launches: keys own (dK, dV), then queries own (dQ).
 void launch(const Args& a, uint64_t units, bool bf16, hipStream_t stream);

@@ -88,13 +88,13 @@ struct KParams {
   float scale;
 };
 
-// T: element type; HP: head size padded to 64 or 128; OWNER_K: the work-group owns keys (else queries).
+// T: element type; HP: head size padded to 64, 128 or 256 (one wave per SIMD at 256); OWNER_K: the work-group owns keys (else queries).
 // DS: accumulate out1 from dS (dK or dQ); PV: accumulate out2 from P (dV, owner = keys).  The
 // keys-own work is run as two launches, one per output: with both accumulator sets and both owner
 // operands a wave needs more than half the register file, and one wave per SIMD cannot overlap its
 // matrix and vector work; recomputing S in a second launch at two waves per SIMD is faster.
 template <typename T, int HP, bool OWNER_K, bool CAUSAL, bool DS, bool PV>
-__global__ __launch_bounds__(256, 2) void fmha_bwd_kernel(KParams p) {
+__global__ __launch_bounds__(256, HP <= 128 ? 2 : 1) void fmha_bwd_kernel(KParams p) {
   static_assert(DS || PV, "nothing to compute");
   static_assert(!PV || OWNER_K, "P^T dO belongs to the keys-own pass");
   typedef typename Elem<T>::vec8 V8;
@@ -386,17 +386,19 @@ void launch_both(const fmha_bwd_fused::Args& a, uint64_t units, hipStream_t st) 
 namespace fmha_bwd_fused {
 
 bool eligible(const Args& a, uint64_t units) {
-  return a.H <= 128 && a.H % 8 == 0 && units * ((uint64_t)((a.F > a.T ? a.F : a.T) + BO - 1) / BO) < 0x7fffffffull &&
+  return a.H <= 256 && a.H % 8 == 0 && units * ((uint64_t)((a.F > a.T ? a.F : a.T) + BO - 1) / BO) < 0x7fffffffull &&
          (uint64_t)a.F * a.H * 2 < kOob && (uint64_t)a.T * a.H * 2 < kOob;
 }
 
 void launch(const Args& a, uint64_t units, bool bf16, hipStream_t st) {
   if (bf16) {
     if (a.H <= 64) launch_both<__bf16, 64>(a, units, st);
-    else launch_both<__bf16, 128>(a, units, st);
+    else if (a.H <= 128) launch_both<__bf16, 128>(a, units, st);
+    else launch_both<__bf16, 256>(a, units, st);
   } else {
     if (a.H <= 64) launch_both<_Float16, 64>(a, units, st);
-    else launch_both<_Float16, 128>(a, units, st);
+    else if (a.H <= 128) launch_both<_Float16, 128>(a, units, st);
+    else launch_both<_Float16, 256>(a, units, st);
   }
 }
 

@@ -7,8 +7,8 @@ mantissa bits fewer) for bf16.  P, dS and the forward output O (which enters thr
 D = rowsum(dO o O)) are rounded to the 16-bit operand type before the products that consume them,
 here as in the reference (xetla/sdp/fmha_backward.h:195-196); the measured elementwise error is
 rounding-dominated: <= 0.4 % for fp16 and <= 5.4 % for bf16 (largest under a causal mask, where late
-keys receive few terms), the same for the fused kernels (no bias, head size <= 128) and for the GEMM
-composition (bias or larger heads; XMK_FMHA_BWD_COMPOSED=1 forces it); the shapes below cover both.  The reference's own attention test allows atol 3e-2 for
+keys receive few terms), the same for the fused kernels (no bias) and for the GEMM
+composition (with a bias; XMK_FMHA_BWD_COMPOSED=1 forces it); the shapes below cover both.  The reference's own attention test allows atol 3e-2 for
 bf16 and 1e-2 for fp16 on O(1) outputs (test/jax_ut.patch:997)."""
 import numpy as np
 import pytest
