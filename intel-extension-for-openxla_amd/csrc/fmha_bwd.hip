@@ -1,5 +1,5 @@
-// Multi-head attention backward: entry point, D = rowsum(dO o O), and the path for what the fused
-// kernels (fmha_bwd_fused.hip: no bias) do not take -- a composition of the batched
+// Multi-head attention backward: entry point, D = rowsum(dO o O), and the second implementation beside
+// the fused kernels (fmha_bwd_fused.hip), selected with XMK_FMHA_BWD_COMPOSED=1 -- a composition of the batched
 // MFMA GEMM and two elementwise passes over the score matrix, for a chunk of (batch, head) units at a time:
 //     D   = rowsum(dO o O)                          (dp_sum, fmha_backward.h:48)
 //     S   = Q K^T                    fp32           (GEMM)
@@ -128,12 +128,12 @@ int run(const void* q, const void* k, const void* v, const void* bias, const voi
   const int64_t rows = units * F;
   hipLaunchKernelGGL(dp_sum_kernel<T>, dim3((unsigned)xmk::ceil_div(rows, 4)), dim3(256), 0, st, (const T*)o, dO,
                      dsum, rows, (int)H);
-  // Without a bias the gradients come from the fused kernels, which
-  // keep the scores on chip; XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
+  // The gradients come from the fused kernels, which keep the scores on chip;
+  // XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
   {
     static const bool composed = getenv("XMK_FMHA_BWD_COMPOSED") != nullptr;
-    const fmha_bwd_fused::Args a{q, k, v, d_o, lse, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
-    if (!bias && !composed && fmha_bwd_fused::eligible(a, (uint64_t)units)) {
+    const fmha_bwd_fused::Args a{q, k, v, d_o, bias, lse, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
+    if (!composed && fmha_bwd_fused::eligible(a, (uint64_t)units)) {
       fmha_bwd_fused::launch(a, (uint64_t)units, dtype == XMK_BF16, st);
       return xmk::check_launch("fmha_bwd");
     }

@@ -12,6 +12,7 @@ struct Args {
   const void* k;
   const void* v;
   const void* d_o;
+  const void* bias;   // [units, F, T] additive bias or null
   const float* lse;   // [units, F] log-sum-exp of the forward pass (natural log)
   const float* dsum;  // [units, F] rowsum(dO o O)
   void* dq;
@@ -22,7 +23,7 @@ struct Args {
   bool causal;
 };
 
-// Head sizes up to 256 (multiples of 8), no additive bias.
+// Head sizes up to 256 (multiples of 8); a bias of at most 2 GiB per unit.
 bool eligible(const Args& a, uint64_t units);
 // Two launches: keys own (dK, dV), then queries own (dQ).
 void launch(const Args& a, uint64_t units, bool bf16, hipStream_t stream);

@@ -78,6 +78,8 @@ struct KParams {
   const void* own2;   // owner operand of the dP product:      V (owner = keys) or dO
   const void* strm1;  // streamed operand of the score product: Q (owner = keys) or K
   const void* strm2;  // streamed operand of the dP product:    dO (owner = keys) or V
+  const void* bias;   // [units, F, T] additive bias of the scores, or null
+  int bias_vec;       // queries-own pass: the bias may be read 4 keys (8 bytes) at a time
   const float* lse;   // [units, F] natural-log LSE of the forward pass
   const float* dsum;  // [units, F] D = rowsum(dO o O)
   void* out1;         // scale * dS^T Q (dK)  or  scale * dS K (dQ)
@@ -93,8 +95,11 @@ struct KParams {
 // keys-own work is run as two launches, one per output: with both accumulator sets and both owner
 // operands a wave needs more than half the register file, and one wave per SIMD cannot overlap its
 // matrix and vector work; recomputing S in a second launch at two waves per SIMD is faster.
-template <typename T, int HP, bool OWNER_K, bool CAUSAL, bool DS, bool PV>
-__global__ __launch_bounds__(256, HP <= 128 ? 2 : 1) void fmha_bwd_kernel(KParams p) {
+// BIAS: S + bias enters the softmax; the bias is read from global memory at the start of each block
+// (keys-own pass: 2-byte loads that are contiguous across the lanes of a wave; queries-own pass: each
+// lane reads its own row, 8 bytes at a time where the alignment allows).
+template <typename T, int HP, bool OWNER_K, bool CAUSAL, bool DS, bool PV, bool BIAS>
+__global__ __launch_bounds__(256, (HP <= 128 && !BIAS) ? 2 : 1) void fmha_bwd_kernel(KParams p) {
   static_assert(DS || PV, "nothing to compute");
   static_assert(!PV || OWNER_K, "P^T dO belongs to the keys-own pass");
   typedef typename Elem<T>::vec8 V8;
@@ -220,6 +225,42 @@ __global__ __launch_bounds__(256, HP <= 128 ? 2 : 1) void fmha_bwd_kernel(KParam
 #pragma unroll
   for (int i = 0; i < (PV ? HT : 1); ++i) acc2[i] = zero16();
   const float scale2 = p.scale * kLog2e;
+  auto to_f32 = [](uint16_t b) -> float {
+    if constexpr (sizeof(T) == 2 && __is_same(T, __bf16)) return __builtin_bit_cast(float, (uint32_t)b << 16);
+    else return (float)__builtin_bit_cast(_Float16, b);
+  };
+  // Bias of one block in the layout of the scores: bs[kt][i] <-> streamed row t0 + 32 kt + 8 (i/4) + 4 g + i%4.
+  auto load_bias = [&](int t0, float (&bs)[2][16]) {
+    const T* bb = reinterpret_cast<const T*>(p.bias) + (int64_t)unit * p.F * p.T;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(bb, (uint32_t)((int64_t)p.F * p.T * 2));
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int s0 = t0 + 32 * kt + 8 * qd + 4 * g;  // first of 4 streamed rows
+        if constexpr (OWNER_K) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int q = s0 + e;
+            const uint32_t off = (q < p.F && orow < p.T) ? (uint32_t)(((int64_t)q * p.T + orow) * 2) : kOob;
+            bs[kt][4 * qd + e] = to_f32((uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0));
+          }
+        } else {
+          if (p.bias_vec) {  // T % 4 == 0: the 4 keys are inside the row or outside as a whole
+            const uint32_t off = (orow < p.F && s0 < p.T) ? (uint32_t)(((int64_t)orow * p.T + s0) * 2) : kOob;
+            const u32x2 w = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bs[kt][4 * qd + e] = to_f32((uint16_t)(w[e >> 1] >> (16 * (e & 1))));
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const uint32_t off = (orow < p.F && s0 + e < p.T) ? (uint32_t)(((int64_t)orow * p.T + s0 + e) * 2) : kOob;
+              bs[kt][4 * qd + e] = to_f32((uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0));
+            }
+          }
+        }
+      }
+  };
 
   // Blocks of streamed rows this work-group needs.
   //   owner = queries, causal: keys up to its last query.   owner = keys, causal: queries from its first key on.
@@ -271,6 +312,8 @@ __global__ __launch_bounds__(256, HP <= 128 ? 2 : 1) void fmha_bwd_kernel(KParam
       issue_tile(Str2, t0 + BS, n2);
       if constexpr (OWNER_K) issue_stats(t0 + BS, nst);
     }
+    float bs[BIAS ? 2 : 1][16];
+    if constexpr (BIAS) load_bias(t0, bs);
     floatx16 sc[2], dp[2];
     scores(c1, of1, sc);
     if constexpr (DS) scores(c2, of2, dp);
@@ -295,7 +338,11 @@ __global__ __launch_bounds__(256, HP <= 128 ? 2 : 1) void fmha_bwd_kernel(KParam
             const int i = 4 * qd + e;
             const float lse2 = OWNER_K ? l2[e] * kLog2e : own_lse2;
             const float dq = OWNER_K ? dd[e] : own_d;
-            float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, -lse2));
+            float pr;
+            if constexpr (BIAS)
+              pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, __builtin_fmaf(bs[kt][i], kLog2e, -lse2)));
+            else
+              pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, -lse2));
             if constexpr (MASKED) {
               const int srow = t0 + 32 * kt + 8 * qd + 4 * g + e;
               const int q = OWNER_K ? srow : orow;
@@ -363,14 +410,21 @@ void launch_pass(KParams p, uint64_t units, bool causal, hipStream_t st) {
   p.total = (int)(units * p.nob);
   p.per_xcd = (p.total + 7) / 8;
   const dim3 grid((unsigned)(p.per_xcd * 8)), block(256);
-  if (causal) hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, true, DS, PV>), grid, block, 0, st, p);
-  else hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, false, DS, PV>), grid, block, 0, st, p);
+  if (p.bias) {
+    if (causal) hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, true, DS, PV, true>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, false, DS, PV, true>), grid, block, 0, st, p);
+  } else {
+    if (causal) hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, true, DS, PV, false>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, false, DS, PV, false>), grid, block, 0, st, p);
+  }
 }
 
 template <typename T, int HP>
 void launch_both(const fmha_bwd_fused::Args& a, uint64_t units, hipStream_t st) {
   KParams p;
   p.lse = a.lse; p.dsum = a.dsum; p.H = a.H; p.F = a.F; p.T = a.T; p.scale = a.scale;
+  p.bias = a.bias;
+  p.bias_vec = a.bias && a.T % 4 == 0 && xmk::aligned(a.bias, 8);
   p.nob = p.total = p.per_xcd = 0;
   // owner = keys: dK, then dV
   p.own1 = a.k; p.own2 = a.v; p.strm1 = a.q; p.strm2 = a.d_o; p.out1 = a.dk; p.out2 = a.dv;
@@ -387,7 +441,8 @@ namespace fmha_bwd_fused {
 
 bool eligible(const Args& a, uint64_t units) {
   return a.H <= 256 && a.H % 8 == 0 && units * ((uint64_t)((a.F > a.T ? a.F : a.T) + BO - 1) / BO) < 0x7fffffffull &&
-         (uint64_t)a.F * a.H * 2 < kOob && (uint64_t)a.T * a.H * 2 < kOob;
+         (uint64_t)a.F * a.H * 2 < kOob && (uint64_t)a.T * a.H * 2 < kOob &&
+         (!a.bias || (uint64_t)a.F * a.T * 2 < kOob);
 }
 
 void launch(const Args& a, uint64_t units, bool bf16, hipStream_t st) {

@@ -7,8 +7,8 @@ mantissa bits fewer) for bf16.  P, dS and the forward output O (which enters thr
 D = rowsum(dO o O)) are rounded to the 16-bit operand type before the products that consume them,
 here as in the reference (xetla/sdp/fmha_backward.h:195-196); the measured elementwise error is
 rounding-dominated: <= 0.4 % for fp16 and <= 5.4 % for bf16 (largest under a causal mask, where late
-keys receive few terms), the same for the fused kernels (no bias) and for the GEMM
-composition (with a bias; XMK_FMHA_BWD_COMPOSED=1 forces it); the shapes below cover both.  The reference's own attention test allows atol 3e-2 for
+keys receive few terms), the same for the fused kernels and for the GEMM
+composition (XMK_FMHA_BWD_COMPOSED=1, which test_backward_composition runs in a child process).  The reference's own attention test allows atol 3e-2 for
 bf16 and 1e-2 for fp16 on O(1) outputs (test/jax_ut.patch:997)."""
 import numpy as np
 import pytest
@@ -54,12 +54,40 @@ def test_backward_shapes(xmk, oracle, name, causal, use_bias, F, T, H):
     _run(xmk, oracle, name, 2, 3, F, T, H, causal, use_bias)
 
 
-def test_backward_chunks_over_units(xmk, oracle):
-    """More units than fit one workspace chunk (score buffers are capped at 1 GiB).  The maximum
-    over 1.5 M elements of a rounding-dominated error sits further out in the tail than on the
-    small shapes, so the elementwise bound is wider here; the scale-relative bound is the same."""
+def test_backward_large(xmk, oracle):
+    """Many blocks with a bias and a causal mask.  The maximum over 1.5 M elements of a
+    rounding-dominated error sits further out in the tail than on the small shapes, so the
+    elementwise bound is wider here; the scale-relative bound is the same."""
     errs = _run(xmk, oracle, "bf16", 1, 12, 2048, 2048, 64, True, True, seed=9, tol_elem=1e-1)
     print(errs)
+
+
+_COMPOSED_CHILD = """
+import sys
+sys.path.insert(0, {tests!r}); sys.path.insert(0, {root!r})
+import importlib
+import oracle
+import test_fmha_bwd_gpu as t
+xmk = importlib.import_module("intel-extension-for-openxla_amd")
+t._run(xmk, oracle, "fp16", 2, 3, 200, 136, 128, True, True)
+t._run(xmk, oracle, "bf16", 2, 3, 257, 64, 256, False, False)
+# more units than fit one workspace chunk (score buffers are capped at 1 GiB)
+t._run(xmk, oracle, "bf16", 1, 12, 2048, 2048, 64, True, False, seed=9, tol_elem=1e-1)
+print("composed ok")
+"""
+
+
+def test_backward_composition():
+    """The GEMM composition (the path behind XMK_FMHA_BWD_COMPOSED=1) in a child process, since the
+    switch is read once per process: bias, head size 256, and chunking over units."""
+    import os
+    import subprocess
+    import sys
+    tests = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ, XMK_FMHA_BWD_COMPOSED="1")
+    r = subprocess.run([sys.executable, "-c", _COMPOSED_CHILD.format(tests=tests, root=os.path.dirname(tests))],
+                       env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "composed ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
 @pytest.mark.parametrize("name,causal", [("bf16", True), ("fp16", False)])
