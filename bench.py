@@ -80,6 +80,20 @@ def wl_fmha(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
                 note="causal FLOPs counted as 2*B*N*S^2*D (half of the dense 4*B*N*S^2*D)")
 
 
+def wl_fmha_bwd(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
+    """Gradients of the headline attention shape.  Flops counted as the 5 products of the textbook
+    backward (2.5x the forward's), although the kernels recompute S per pass."""
+    q, k, v, d_o = (torch.randn((B, N, S, H), device="cuda").bfloat16() for _ in range(4))
+    out = torch.empty_like(q)
+    lse = torch.empty((B * N, S), dtype=torch.float32, device="cuda")
+    xmk.fmha_forward(q, k, v, out, lse=lse, causal=causal)
+    flops = 10.0 * B * N * S * S * H * (0.5 if causal else 1.0)
+    return dict(name=f"fmha_bwd_{'causal_' if causal else ''}bf16_b{B}_h{N}_s{S}_d{H}",
+                fn=lambda: xmk.fmha_backward(q, k, v, out, d_o, lse, causal=causal), flops=flops,
+                bytes=10.0 * B * N * S * H * 2, bound="mfma", dtype="bf16", kernel="fmha_bwd_kernel (3 launches)",
+                note="flops counted as 5 matrix products (2.5x forward)")
+
+
 def wl_gemm(torch, xmk, m, n, k, bias=False, rhs_t=False):
     a = (torch.randn((m, k), device="cuda") * k ** -0.5).bfloat16()
     b = (torch.randn((n, k) if rhs_t else (k, n), device="cuda") * k ** -0.5).bfloat16()
@@ -186,6 +200,8 @@ WORKLOADS = {
     "mfma_probe_fp8_16": lambda t, x: wl_mfma_probe(t, x, 16, fp8=True),
     "fmha_causal": lambda t, x: wl_fmha(t, x, True),
     "fmha": lambda t, x: wl_fmha(t, x, False),
+    "fmha_bwd_causal": lambda t, x: wl_fmha_bwd(t, x, True),
+    "fmha_bwd": lambda t, x: wl_fmha_bwd(t, x, False),
     "gemm_8192": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192),
     "gemm_8192_rhsT": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192, rhs_t=True),
     "gemm_c1": lambda t, x: wl_gemm(t, x, 512, 4096, 4096, bias=True),
@@ -195,7 +211,7 @@ WORKLOADS = {
     "fp8_8192": lambda t, x: wl_fp8(t, x, 8192, 8192, 8192),
     "gptj_decode": lambda t, x: wl_gptj_decode(t, x),
 }
-ALSO = ["gemm_8192", "gemm_8192_rhsT", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "gptj_decode",
+ALSO = ["fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "gptj_decode",
         "mfma_probe_32", "mfma_probe_16", "mfma_probe_fp8_32", "mfma_probe_fp8_16"]
 
 

@@ -21,18 +21,28 @@ namespace {
 
 constexpr size_t kChunkBytes = (size_t)1 << 30;  // score-sized intermediates per chunk, at most
 
-template <typename T>
+// D[row] = sum_h O[row][h] dO[row][h].  H % 8 == 0: a lane reads 8 elements (16 bytes) of each tensor;
+// LPR lanes (a power of two >= H / 8) share a row and a wave covers 64 / LPR rows.
+template <typename T, int LPR>
 __global__ __launch_bounds__(256) void dp_sum_kernel(const T* __restrict__ o, const T* __restrict__ d_o,
                                                      float* __restrict__ dsum, int64_t rows, int H) {
-  // one wave per row
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63;
+  const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPR;
+  const int c = (lane % LPR) * 8;
   float s = 0.f;
-  for (int h = lane; h < H; h += 64) s += (float)o[row * H + h] * (float)d_o[row * H + h];
+  if (row < rows && c < H) {
+    const u32x4 a = *reinterpret_cast<const u32x4*>(o + row * H + c);
+    const u32x4 b = *reinterpret_cast<const u32x4*>(d_o + row * H + c);
+    const T* ae = reinterpret_cast<const T*>(&a);
+    const T* be = reinterpret_cast<const T*>(&b);
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off);
-  if (lane == 0) dsum[row] = s;
+    for (int j = 0; j < 8; ++j) s += (float)ae[j] * (float)be[j];
+  }
+#pragma unroll
+  for (int off = LPR / 2; off >= 1; off >>= 1) s += __shfl_xor(s, off);
+  if (row < rows && lane % LPR == 0) dsum[row] = s;
 }
 
 // P[u, f, t] = exp(scale * S + bias - lse[f]); masked entries (causal: t > f) are zero.
@@ -126,8 +136,15 @@ int run(const void* q, const void* k, const void* v, const void* bias, const voi
   const T* Q = (const T*)q; const T* K = (const T*)k; const T* V = (const T*)v; const T* dO = (const T*)d_o;
   T* dQ = (T*)dq; T* dK = (T*)dk; T* dV = (T*)dv;
   const int64_t rows = units * F;
-  hipLaunchKernelGGL(dp_sum_kernel<T>, dim3((unsigned)xmk::ceil_div(rows, 4)), dim3(256), 0, st, (const T*)o, dO,
-                     dsum, rows, (int)H);
+  if (H <= 64)
+    hipLaunchKernelGGL((dp_sum_kernel<T, 8>), dim3((unsigned)xmk::ceil_div(rows, 32)), dim3(256), 0, st, (const T*)o, dO,
+                       dsum, rows, (int)H);
+  else if (H <= 128)
+    hipLaunchKernelGGL((dp_sum_kernel<T, 16>), dim3((unsigned)xmk::ceil_div(rows, 16)), dim3(256), 0, st, (const T*)o, dO,
+                       dsum, rows, (int)H);
+  else
+    hipLaunchKernelGGL((dp_sum_kernel<T, 32>), dim3((unsigned)xmk::ceil_div(rows, 8)), dim3(256), 0, st, (const T*)o, dO,
+                       dsum, rows, (int)H);
   // The gradients come from the fused kernels, which keep the scores on chip;
   // XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
   {
