@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also] [--no-cpu]
 
 One JSON line on stdout.  A "step" is one launch of the workload's kernel on synthetic inputs that
-are already resident in HBM.  The headline workload is BASELINE config 2 (fused causal MHA forward,
+are already resident in HBM.  The headline workload is benchmark configuration 2 (fused causal MHA forward,
 bf16 [8,32,2048,128]); the other configs are timed the same way and reported under "also".
 """
 import argparse
@@ -139,7 +139,7 @@ def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
 
 
 def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
-    """BASELINE config 5: GPT-J-6B-shaped decode step, int4 group-128 weights, fp16 KV cache filled to
+    """benchmark configuration 5: GPT-J-6B-shaped decode step, int4 group-128 weights, fp16 KV cache filled to
     `cache_len`, one new token per sequence.  The whole step (about 8 launches per block) is replayed
     from one HIP graph."""
     d, heads, hd, dff, vocab, g = 4096, 16, 256, 16384, 50400, 128

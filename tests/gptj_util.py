@@ -23,7 +23,7 @@ def load_fixture(oracle):
 
 
 def random_model(oracle, cfg, seed=0):
-    """Random int4 model as bit patterns, inputs as BASELINE config 5 describes them."""
+    """Random int4 model as bit patterns, inputs as benchmark configuration 5 describes them."""
     d, dff, V, g = cfg["d_model"], cfg["d_ff"], cfg["vocab"], cfg["group"]
 
     def lin(k, n, s, bias):

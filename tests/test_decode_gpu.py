@@ -62,7 +62,7 @@ def test_gptj_tiny_matches_transformers_fixture(xmk, oracle):
 
 @pytest.mark.parametrize("n_layer,position", [(2, 2047), (1, 0), (1, 300)])
 def test_gptj_full_width_vs_oracle(xmk, oracle, n_layer, position):
-    """BASELINE config 5 at full width (d_model 4096, 16 heads x 256, rotary 64, MLP 16384, vocab
+    """benchmark configuration 5 at full width (d_model 4096, 16 heads x 256, rotary 64, MLP 16384, vocab
     50400, batch 4, cache filled with N(0,1) to `position`), fewer blocks so the numpy oracle
     finishes in seconds."""
     from oracle import gptj as og

@@ -45,7 +45,7 @@ def _run(xmk, oracle, name, B, N, F, T, H, *, causal=False, use_bias=False, lse=
 
 
 def test_config2_causal_bf16(xmk, oracle):
-    """BASELINE config 2: bf16 [8,32,2048,128], causal, scale 1/sqrt(128); three units, every 8th row."""
+    """benchmark configuration 2: bf16 [8,32,2048,128], causal, scale 1/sqrt(128); three units, every 8th row."""
     _run(xmk, oracle, "bf16", 8, 32, 2048, 2048, 128, causal=True, units=[0, 101, 255], f_stride=8)
 
 

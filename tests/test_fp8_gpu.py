@@ -35,7 +35,7 @@ def test_fp8_gemm_shapes(xmk, oracle, m, n, k, rhs_t):
 
 
 def test_config4_fp8_8192_sampled_rows(xmk, oracle):
-    """BASELINE config 4: A, B [8192,8192] e4m3fn from N(0,1) with amax/448 scales, bf16 output."""
+    """benchmark configuration 4: A, B [8192,8192] e4m3fn from N(0,1) with amax/448 scales, bf16 output."""
     n = 8192
     a, sa = _quant(oracle, (n, n), 11)
     b, sb = _quant(oracle, (n, n), 12)  # stored [N, K]

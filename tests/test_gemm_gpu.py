@@ -1,6 +1,6 @@
 """GPU parity: bf16/fp16 GEMM with fused epilogue through the C ABI (xmk_gemm), against the oracle.
 
-Tolerance (BASELINE north star): max relative error <= 1e-2 for bf16/fp16 outputs against an
+Tolerance (the tolerance stated for this path): max relative error <= 1e-2 for bf16/fp16 outputs against an
 fp32 recompute from the same rounded inputs; both normalisations of oracle.rel_err are held to it.
 """
 import numpy as np
@@ -25,7 +25,7 @@ def _check(oracle, got_f32, ref_f32, tol=TOL):
 
 
 def test_config1_bf16_bias(xmk, oracle):
-    """BASELINE config 1: C[512,4096] = A[512,4096] B[4096,4096] + bias, N(0,1)/sqrt(K) inputs."""
+    """benchmark configuration 1: C[512,4096] = A[512,4096] B[4096,4096] + bias, N(0,1)/sqrt(K) inputs."""
     m, k, n = 512, 4096, 4096
     sc = k ** -0.5
     a = oracle.from_f32(oracle.normal((m, k), 1, sc), oracle.BF16)

@@ -28,7 +28,7 @@ def test_int4_dequant_bit_exact(xmk, oracle, k, n, group):
 
 @pytest.mark.parametrize("m", [1, 8, 32])
 def test_int4_gemm_gptj_mlp_shape(xmk, oracle, m):
-    """BASELINE config 3: K=4096, N=16384, group 128, M in {1, 8, 32}; <= 1e-2 vs fp32 recompute."""
+    """benchmark configuration 3: K=4096, N=16384, group 128, M in {1, 8, 32}; <= 1e-2 vs fp32 recompute."""
     k, n, group = 4096, 16384, 128
     act, qw, s, z = _case(oracle, m, k, n, group, 7)
     _, ref = oracle.int4_gemm(act, qw, s, z, group)
