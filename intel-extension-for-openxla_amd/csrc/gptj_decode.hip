@@ -41,13 +41,23 @@ __global__ __launch_bounds__(LN_NT) void layernorm_kernel(const _Float16* __rest
         float f[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) f[e] = (float)v[j].e[e];
+        // All slices are loaded before the first is added: with four work-groups in the whole launch
+        // the chain of load latencies is what this kernel costs.  Added in slice order.
         auto add_slices = [&](const float* p, int ks) {
-          for (int sl = 0; sl < ks; ++sl) {
-            const float* q = p + ((size_t)sl * 32 + blockIdx.x) * d + i;
-            const ln_f32x4 lo = *reinterpret_cast<const ln_f32x4*>(q), hi = *reinterpret_cast<const ln_f32x4*>(q + 4);
+          ln_f32x4 lo[xmk::kInt4MaxSplit], hi[xmk::kInt4MaxSplit];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { f[e] += lo[e]; f[4 + e] += hi[e]; }
-          }
+          for (int sl = 0; sl < xmk::kInt4MaxSplit; ++sl)
+            if (sl < ks) {
+              const float* q = p + ((size_t)sl * 32 + blockIdx.x) * d + i;
+              lo[sl] = *reinterpret_cast<const ln_f32x4*>(q);
+              hi[sl] = *reinterpret_cast<const ln_f32x4*>(q + 4);
+            }
+#pragma unroll
+          for (int sl = 0; sl < xmk::kInt4MaxSplit; ++sl)
+            if (sl < ks) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) { f[e] += lo[sl][e]; f[4 + e] += hi[sl][e]; }
+            }
         };
         add_slices(p1, ks1);
         add_slices(p2, ks2);
