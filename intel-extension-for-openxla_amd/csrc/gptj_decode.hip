@@ -1,6 +1,6 @@
-// GPT-J-shaped decode step on int4 weights: the glue kernels (LayerNorm, rotary embedding
-// fused with the KV-cache append) and the host loop that strings them together with the
-// int4 GEMM and the split-key decode attention.  Everything is enqueued on one stream, in
+// GPT-J-shaped decode step on int4 weights: the LayerNorm kernel and the host loop that strings it
+// together with the int4 GEMM (whose q/k/v epilogue applies the rotary embedding and appends to the
+// KV cache) and the split-key decode attention.  Everything is enqueued on one stream, in
 // order, with no host synchronisation, so a caller can capture the whole step in a HIP graph.
 #include "common.h"
 #include "int4_gemm.h"
@@ -111,43 +111,6 @@ __global__ __launch_bounds__(LN_NT) void layernorm_kernel(const _Float16* __rest
         o.e[e] = (_Float16)(((float)v[j].e[e] - mean) * rstd * (float)g.e[e] + (float)b.e[e]);
       *reinterpret_cast<ln_u32x4*>(y + (size_t)blockIdx.x * d + i) = o.u;
     }
-  }
-}
-
-// qkv [B, 3 d] (columns q | k | v, head-major).  Rotates the first rotary_dim dims of every q
-// and k head (interleaved pairs, angle = position * 10000^(-2i/rotary_dim)); writes q to
-// q_out [B, d], and k (rotated) and v to row `position` of the caches [B, N, cap, H].
-__global__ __launch_bounds__(256) void rope_append_kernel(const _Float16* __restrict__ qkv,
-                                                          _Float16* __restrict__ q_out,
-                                                          _Float16* __restrict__ k_cache,
-                                                          _Float16* __restrict__ v_cache, int n_head,
-                                                          int head_dim, int rotary_dim, int cap,
-                                                          int position) {
-  const int b = blockIdx.y, head = blockIdx.x;
-  const int d = n_head * head_dim;
-  const _Float16* q = qkv + (size_t)b * 3 * d + (size_t)head * head_dim;
-  const _Float16* k = q + d;
-  const _Float16* v = q + 2 * d;
-  _Float16* qo = q_out + (size_t)b * d + (size_t)head * head_dim;
-  const size_t crow = (((size_t)b * n_head + head) * cap + position) * head_dim;
-  for (int i = threadIdx.x; i < head_dim / 2; i += 256) {
-    float q0 = (float)q[2 * i], q1 = (float)q[2 * i + 1];
-    float k0 = (float)k[2 * i], k1 = (float)k[2 * i + 1];
-    if (2 * i < rotary_dim) {
-      const float inv_freq = powf(10000.0f, -(float)(2 * i) / (float)rotary_dim);
-      float sn, cs;
-      sincosf((float)position * inv_freq, &sn, &cs);
-      const float a = q0 * cs - q1 * sn, bq = q1 * cs + q0 * sn;
-      q0 = a; q1 = bq;
-      const float c = k0 * cs - k1 * sn, dk = k1 * cs + k0 * sn;
-      k0 = c; k1 = dk;
-    }
-    qo[2 * i] = (_Float16)q0;
-    qo[2 * i + 1] = (_Float16)q1;
-    k_cache[crow + 2 * i] = (_Float16)k0;
-    k_cache[crow + 2 * i + 1] = (_Float16)k1;
-    v_cache[crow + 2 * i] = v[2 * i];
-    v_cache[crow + 2 * i + 1] = v[2 * i + 1];
   }
 }
 
@@ -281,12 +244,14 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
     xmk::Int4Epilogue gelu;
     gelu.gelu = 1;
     xmk::Int4Call c_qkv, c_fc_in, c_out, c_fc_out;
-    if ((rc = make_call(L.qkv, w.h, w.qkv, d, 3 * d, xmk::Int4Epilogue{}, "qkv", &c_qkv)) != XMK_OK) return rc;
+    // The q/k/v product applies the rotary embedding and appends k and v to the caches in its epilogue.
+    xmk::Int4Epilogue rope;
+    rope.rope_d = (int)d; rope.head_dim = c.head_dim; rope.rotary_dim = c.rotary_dim;
+    rope.capacity = c.cache_capacity; rope.position = position;
+    rope.q_out = w.q; rope.k_cache = L.k_cache; rope.v_cache = L.v_cache;
+    if ((rc = make_call(L.qkv, w.h, w.qkv, d, 3 * d, rope, "qkv", &c_qkv)) != XMK_OK) return rc;
     if ((rc = make_call(L.fc_in, w.h, w.ff, d, dff, gelu, "fc_in", &c_fc_in)) != XMK_OK) return rc;
     if ((rc = xmk::int4_gemm_launch2(c_qkv, &c_fc_in, B, c.group, st)) != XMK_OK) return rc;
-    hipLaunchKernelGGL(rope_append_kernel, dim3((unsigned)c.n_head, (unsigned)B), dim3(256), 0, st, w.qkv, w.q,
-                       (_Float16*)L.k_cache, (_Float16*)L.v_cache, c.n_head, c.head_dim, c.rotary_dim,
-                       c.cache_capacity, position);
     if ((rc = xmk_fmha_decode(w.q, L.k_cache, L.v_cache, w.attn, XMK_F16, (uint32_t)B, (uint32_t)c.n_head,
                               (uint32_t)c.head_dim, (uint32_t)(position + 1), head_stride, scale, w.attn_ws,
                               w.attn_ws_bytes, stream)) != XMK_OK)
@@ -303,7 +268,7 @@ extern "C" int xmk_gptj_decode_step(const xmk_gptj_config* cfg, const xmk_gptj_l
       pending = true;
       pending_bias = (const _Float16*)L.fc_out.bias;
     } else {
-      // out_proj result goes to w.qkv's first B*d elements (qkv is dead after the rotary kernel);
+      // out_proj result goes to w.qkv's first B*d elements (the q/k/v product writes q and the caches, not this buffer);
       // fc_out adds bias, the residual x and the attention branch in its epilogue
       _Float16* a_out = w.qkv;
       if ((rc = make_call(L.out_proj, w.attn, a_out, d, d, xmk::Int4Epilogue{}, "out_proj", &c_out)) != XMK_OK) return rc;

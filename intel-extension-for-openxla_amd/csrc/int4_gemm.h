@@ -12,6 +12,16 @@ struct Int4Epilogue {
   int gelu = 0;
   const void* add0 = nullptr;
   const void* add1 = nullptr;
+  // rope_d > 0: the product is a stacked q/k/v projection [rows, 3 * rope_d] of one decode step
+  // (rope_d = heads * head_dim).  Instead of being stored to `out`, q and k get the GPT-J rotary
+  // embedding (interleaved pairs of the first rotary_dim elements of each head, angle = position *
+  // 10000^(-2i/rotary_dim)); q goes to q_out [rows, rope_d], k and v to row `position` of the caches
+  // [rows, heads, capacity, head_dim].
+  int rope_d = 0;
+  int head_dim = 0, rotary_dim = 0, capacity = 0, position = 0;
+  void* q_out = nullptr;
+  void* k_cache = nullptr;
+  void* v_cache = nullptr;
 };
 
 // Splitting K over work-groups, for shapes whose N alone gives too few of them.  With

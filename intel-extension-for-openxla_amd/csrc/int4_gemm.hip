@@ -298,6 +298,30 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
 #pragma unroll
     for (int w = 0; w < NW; ++w) s += red[w][row][col];
     if (bias) s += (float)bias[n];
+    if (ep.rope_d > 0) {
+      const int d = ep.rope_d, which = n / d, hd = n % d;  // 0 q, 1 k, 2 v; element of the [heads, head_dim] row
+      const int head = hd / ep.head_dim, i = hd % ep.head_dim;
+      if (which < 2 && i < ep.rotary_dim) {
+        // the other element of the rotary pair sits in the neighbouring column of this block
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) t += red[w][row][col ^ 1];
+        if (bias) t += (float)bias[n ^ 1];
+        const float inv_freq = powf(10000.0f, -(float)(i & ~1) / (float)ep.rotary_dim);
+        float sn, cs;
+        sincosf((float)ep.position * inv_freq, &sn, &cs);
+        s = (i & 1) ? s * cs + t * sn : s * cs - t * sn;
+      }
+      const int m = m_base + row;
+      if (which == 0) {
+        reinterpret_cast<_Float16*>(ep.q_out)[(size_t)m * d + hd] = (_Float16)s;
+      } else {
+        _Float16* cache = reinterpret_cast<_Float16*>(which == 1 ? ep.k_cache : ep.v_cache);
+        const int heads = d / ep.head_dim;
+        cache[(((size_t)m * heads + head) * ep.capacity + ep.position) * ep.head_dim + i] = (_Float16)s;
+      }
+      continue;
+    }
     if (ep.gelu) {  // gelu_new: 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) = x / (1 + e^{-2u})
       const float u = 0.7978845608028654f * (s + 0.044715f * s * s * s);
       s = s / (1.0f + __expf(-2.0f * u));
