@@ -9,6 +9,8 @@
 // output  sum_t 2^(s_t - m) V[t,:]  is written to the workspace together with (m, l).
 // Pass 2 (fmha_decode_merge_kernel): one work-group per unit rescales and adds the
 // partial results and writes the output row.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace {
@@ -214,8 +216,14 @@ __global__ __launch_bounds__(NT) void fmha_decode_merge_kernel(DecodeParams p) {
 }
 
 void plan(uint32_t units, uint32_t T, int* splits, int* chunk) {
-  // About 1024 work-groups in flight, at least 64 and at most 512 keys per chunk.
-  int s = (int)((1024 + units - 1) / units);
+  // About 1024 work-groups in flight (XMK_DECODE_WGS overrides the target), at least 64 and at most
+  // 512 keys per chunk.
+  static const int target = [] {
+    const char* e = getenv("XMK_DECODE_WGS");
+    const int v = e ? atoi(e) : 0;
+    return v >= 64 && v <= 65536 ? v : 1024;
+  }();
+  int s = (int)((target + units - 1) / units);
   int c = (int)((T + s - 1) / s);
   if (c < 64) c = 64;
   if (c > 512) c = 512;
