@@ -228,7 +228,31 @@ typedef struct XLA_FFI_Stream_Get_Args {
 } XLA_FFI_Stream_Get_Args;
 typedef XLA_FFI_Error* XLA_FFI_Stream_Get(XLA_FFI_Stream_Get_Args* args);
 
-/* Leading part of the function table; the entries after Stream_Get are not used here. */
+/* Scratch device memory from the executor's allocator, the C face of ffi::ScratchAllocator
+ * (what the reference's handlers bind with Ctx<ffi::ScratchAllocator>, sycl_custom_call.cc:207-221). */
+typedef struct XLA_FFI_DeviceMemory_Allocate_Args {
+  size_t struct_size;
+  XLA_FFI_Extension_Base* extension_start;
+  XLA_FFI_ExecutionContext* ctx;
+  size_t size;
+  size_t alignment;
+  void* data; /* out */
+} XLA_FFI_DeviceMemory_Allocate_Args;
+typedef XLA_FFI_Error* XLA_FFI_DeviceMemory_Allocate(XLA_FFI_DeviceMemory_Allocate_Args* args);
+
+typedef struct XLA_FFI_DeviceMemory_Free_Args {
+  size_t struct_size;
+  XLA_FFI_Extension_Base* extension_start;
+  XLA_FFI_ExecutionContext* ctx;
+  size_t size;
+  void* data;
+} XLA_FFI_DeviceMemory_Free_Args;
+typedef XLA_FFI_Error* XLA_FFI_DeviceMemory_Free(XLA_FFI_DeviceMemory_Free_Args* args);
+
+/* Leading part of the function table.  The four entries between Stream_Get and
+ * DeviceMemory_Allocate are not used here and kept as opaque pointers; entries after
+ * DeviceMemory_Free are omitted.  A caller's table may be shorter: check struct_size before
+ * touching anything past Stream_Get. */
 struct XLA_FFI_Api {
   size_t struct_size;
   XLA_FFI_Extension_Base* extension_start;
@@ -239,6 +263,12 @@ struct XLA_FFI_Api {
   XLA_FFI_Error_Destroy* XLA_FFI_Error_Destroy;
   XLA_FFI_Handler_Register* XLA_FFI_Handler_Register;
   XLA_FFI_Stream_Get* XLA_FFI_Stream_Get;
+  void* XLA_FFI_TypeId_Register;
+  void* XLA_FFI_ExecutionContext_Get;
+  void* XLA_FFI_State_Set;
+  void* XLA_FFI_State_Get;
+  XLA_FFI_DeviceMemory_Allocate* XLA_FFI_DeviceMemory_Allocate;
+  XLA_FFI_DeviceMemory_Free* XLA_FFI_DeviceMemory_Free;
 };
 
 #ifdef __cplusplus

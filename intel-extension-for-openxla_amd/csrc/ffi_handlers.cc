@@ -4,6 +4,7 @@
 // Host code only: no device work happens here apart from the entry points it calls.
 #include <cmath>
 #include <cstdio>
+#include <cstddef>
 #include <cstring>
 #include <string>
 
@@ -160,6 +161,15 @@ xmk_matrix matrix_from_dict(Frame& fr, const char* who, void* data) {
   return m;
 }
 
+void destroy_error(const XLA_FFI_Api* api, XLA_FFI_Error* e) {
+  if (!api->XLA_FFI_Error_Destroy) return;
+  XLA_FFI_Error_Destroy_Args a;
+  a.struct_size = sizeof(a);
+  a.extension_start = nullptr;
+  a.error = e;
+  api->XLA_FFI_Error_Destroy(&a);
+}
+
 XLA_FFI_Error* gemm_common(XLA_FFI_CallFrame* f, bool lt) {
   if (metadata_query(f) || f->stage != XLA_FFI_ExecutionStage_EXECUTE) return nullptr;
   Frame fr{f};
@@ -194,6 +204,37 @@ XLA_FFI_Error* gemm_common(XLA_FFI_CallFrame* f, bool lt) {
   d.epilogue = epilogue;
   void* stream = fr.stream();
   if (fr.code != XMK_OK) return finish(fr, XMK_OK);
+  // Shapes that gain from a K split take their fp32 partial sums from the executor's scratch allocator
+  // (the reference's handlers hold one too, sycl_custom_call.cc:154-156), when the API table has it.
+  const size_t need = xmk_gemm_workspace_bytes(&d);
+  const XLA_FFI_Api* api = f->api;
+  const bool can_allocate = need > 0 && api &&
+                            api->struct_size >= offsetof(XLA_FFI_Api, XLA_FFI_DeviceMemory_Free) + sizeof(void*) &&
+                            api->XLA_FFI_DeviceMemory_Allocate && api->XLA_FFI_DeviceMemory_Free;
+  if (can_allocate) {
+    XLA_FFI_DeviceMemory_Allocate_Args al;
+    al.struct_size = sizeof(al);
+    al.extension_start = nullptr;
+    al.ctx = f->ctx;
+    al.size = need;
+    al.alignment = 256;
+    al.data = nullptr;
+    XLA_FFI_Error* e = api->XLA_FFI_DeviceMemory_Allocate(&al);
+    if (!e && al.data) {
+      const int rc = xmk_gemm_ws(&d, al.data, need, stream);
+      // Freed in stream order by the executor's allocator: later work on this stream may reuse it.
+      XLA_FFI_DeviceMemory_Free_Args fa;
+      fa.struct_size = sizeof(fa);
+      fa.extension_start = nullptr;
+      fa.ctx = f->ctx;
+      fa.size = need;
+      fa.data = al.data;
+      XLA_FFI_Error* fe = api->XLA_FFI_DeviceMemory_Free(&fa);
+      if (fe) destroy_error(api, fe);
+      return finish(fr, rc);
+    }
+    if (e) destroy_error(api, e);  // no scratch: the unsplit kernel needs none
+  }
   return finish(fr, xmk_gemm(&d, stream));
 }
 

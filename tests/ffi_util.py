@@ -63,7 +63,19 @@ class HandlerRegisterArgs(C.Structure):
                 ("platform", ByteSpan), ("bundle", HandlerBundle), ("traits", C.c_uint32)]
 
 
+class DeviceMemoryAllocateArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("ctx", C.c_void_p),
+                ("size", C.c_size_t), ("alignment", C.c_size_t), ("data", C.c_void_p)]
+
+
+class DeviceMemoryFreeArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("ctx", C.c_void_p),
+                ("size", C.c_size_t), ("data", C.c_void_p)]
+
+
 ERROR_CREATE = C.CFUNCTYPE(C.c_void_p, C.POINTER(ErrorCreateArgs))
+DEVICE_ALLOC = C.CFUNCTYPE(C.c_void_p, C.POINTER(DeviceMemoryAllocateArgs))
+DEVICE_FREE = C.CFUNCTYPE(C.c_void_p, C.POINTER(DeviceMemoryFreeArgs))
 STREAM_GET = C.CFUNCTYPE(C.c_void_p, C.POINTER(StreamGetArgs))
 HANDLER_REGISTER = C.CFUNCTYPE(C.c_void_p, C.POINTER(HandlerRegisterArgs))
 
@@ -72,7 +84,10 @@ class Api(C.Structure):
     _fields_ = [("struct_size", C.c_size_t), ("extension_start", C.c_void_p), ("api_version", ApiVersion),
                 ("internal_api", C.c_void_p), ("XLA_FFI_Error_Create", ERROR_CREATE),
                 ("XLA_FFI_Error_GetMessage", C.c_void_p), ("XLA_FFI_Error_Destroy", C.c_void_p),
-                ("XLA_FFI_Handler_Register", HANDLER_REGISTER), ("XLA_FFI_Stream_Get", STREAM_GET)]
+                ("XLA_FFI_Handler_Register", HANDLER_REGISTER), ("XLA_FFI_Stream_Get", STREAM_GET),
+                ("XLA_FFI_TypeId_Register", C.c_void_p), ("XLA_FFI_ExecutionContext_Get", C.c_void_p),
+                ("XLA_FFI_State_Set", C.c_void_p), ("XLA_FFI_State_Get", C.c_void_p),
+                ("XLA_FFI_DeviceMemory_Allocate", DEVICE_ALLOC), ("XLA_FFI_DeviceMemory_Free", DEVICE_FREE)]
 
 
 class CallFrame(C.Structure):
@@ -90,9 +105,11 @@ class MetadataExtension(C.Structure):
 
 
 class FakeHost:
-    """XLA_FFI_Api with Error_Create, Stream_Get and Handler_Register implemented in Python."""
+    """XLA_FFI_Api with Error_Create, Stream_Get and Handler_Register implemented in Python, and
+    DeviceMemory_Allocate / Free when an ``allocator`` (size, alignment) -> (device pointer, keep-alive
+    object) is given; without one the table ends at Stream_Get, as an older host's would."""
 
-    def __init__(self, stream=0):
+    def __init__(self, stream=0, allocator=None):
         self.errors = []      # (code, message) of every error created
         self.registered = []  # (name, platform, execute pointer)
         self.stream = stream
@@ -112,9 +129,32 @@ class FakeHost:
                                     C.string_at(r.platform.ptr, r.platform.len).decode(), r.bundle.execute))
             return None
 
-        self._cbs = (ERROR_CREATE(error_create), STREAM_GET(stream_get), HANDLER_REGISTER(handler_register))
+        self.allocations = []  # (size, alignment) of every scratch request
+        self.freed = []        # sizes handed back
+        self._live = {}
+
+        def device_alloc(a):
+            r = a.contents
+            ptr, keep = allocator(r.size, r.alignment)
+            self.allocations.append((r.size, r.alignment))
+            self._live[ptr] = keep
+            r.data = ptr
+            return None
+
+        def device_free(a):
+            r = a.contents
+            self.freed.append(r.size)
+            # the tensor is kept until the host object dies: the work that uses it is only enqueued
+            self._keep.append(self._live.pop(r.data, None))
+            return None
+
+        self._cbs = (ERROR_CREATE(error_create), STREAM_GET(stream_get), HANDLER_REGISTER(handler_register),
+                     DEVICE_ALLOC(device_alloc), DEVICE_FREE(device_free))
         self.api = Api()
-        self.api.struct_size = C.sizeof(Api)
+        self.api.struct_size = C.sizeof(Api) if allocator else Api.XLA_FFI_TypeId_Register.offset
+        if allocator:
+            self.api.XLA_FFI_DeviceMemory_Allocate = self._cbs[3]
+            self.api.XLA_FFI_DeviceMemory_Free = self._cbs[4]
         self.api.api_version = ApiVersion(C.sizeof(ApiVersion), None, 0, 1)
         self.api.XLA_FFI_Error_Create = self._cbs[0]
         self.api.XLA_FFI_Stream_Get = self._cbs[1]

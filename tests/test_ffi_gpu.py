@@ -168,3 +168,35 @@ def test_f8_matmul_handler(ffi, oracle):
     _ok(host, ffi.xmk_ffi_cublas_lt_matmul_f8(C.byref(f)))
     g, e = oracle.rel_err(out.float().cpu().numpy(), ref)
     assert g <= 5e-2 and e <= 5e-2, (g, e)
+
+
+def test_gemm_handler_takes_scratch_for_a_k_split(ffi, oracle):
+    """A small-M product with a long reduction: with DeviceMemory_Allocate / Free in the API table the
+    handler asks for exactly xmk_gemm_workspace_bytes of scratch, runs the K-split path and hands the
+    scratch back; with a table that ends at Stream_Get it runs unsplit.  Same result either way."""
+    m, n, k = 4, 4096, 16384
+    a = oracle.from_f32(oracle.normal((m, k), 41, 0.05), oracle.BF16)
+    b = oracle.from_f32(oracle.normal((n, k), 42, 0.05), oracle.BF16)
+    _, ref = oracle.gemm(a, b, oracle.BF16, oracle.BF16, rhs_t=True)
+    da, db = to_dev(a, "bf16"), to_dev(b, "bf16")
+
+    def allocator(size, alignment):
+        t = torch.empty((size + alignment,), dtype=torch.uint8, device="cuda")
+        ptr = (t.data_ptr() + alignment - 1) // alignment * alignment
+        return ptr, t
+
+    outs = []
+    for alloc in (allocator, None):
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        host = F.FakeHost(stream=torch.cuda.current_stream().cuda_stream, allocator=alloc)
+        f = host.frame([_buf(da, F.BF16), _buf(db, F.BF16)], [_buf(out, F.BF16)],
+                       F.gemm_attrs(m, n, k, F.BF16, F.BF16, rhs_col_major=True))
+        _ok(host, ffi.xmk_ffi_cublas_gemm(C.byref(f)))
+        if alloc:
+            assert len(host.allocations) == 1 and host.allocations[0][0] > 0 and host.freed == [host.allocations[0][0]]
+        else:
+            assert host.allocations == []
+        g, e = oracle.rel_err(out.float().cpu().numpy(), ref[0])
+        assert g <= 1e-2 and e <= 1e-2, (g, e)
+        outs.append(out)
+    assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-2
