@@ -16,9 +16,11 @@
 // The products are issued with the operands swapped (D^T = B^T A^T) so that a lane ends up
 // holding four consecutive output columns of one row.
 //
-// Everything the MFMA kernel cannot take (fp32 or int8 operands, unaligned
-// pointers or strides) runs gemm_generic_kernel, a plain LDS-tiled kernel; this is
-// where the reference falls back to oneDNN (onednn_matmul_utils.cc:394-491).
+// 16-bit operands whose strides or sizes the direct loads cannot take run the same kernel with a
+// gathering loader, fp32 operands the fp32 MFMA kernel (gemm_f32.hip); what is left (int8, outputs
+// that are not 16-byte aligned) runs gemm_generic_kernel, a plain LDS-tiled kernel.  This is where
+// the reference falls back to oneDNN (onednn_matmul_utils.cc:394-491).
+#include "gemm_f32.h"
 #include "gemm_kernel.h"
 
 namespace {
@@ -191,6 +193,7 @@ extern "C" const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int
                                             int32_t dtype_in, int32_t dtype_out) {
   (void)rhs_transpose;
   const bool sixteen = dtype_in == XMK_BF16 || dtype_in == XMK_F16;
+  if (dtype_in == XMK_F32 && dtype_out == XMK_F32) return "mfma_f32_128x128x16";
   if (!sixteen || !(dtype_out == dtype_in || dtype_out == XMK_F32)) return "generic_64x64";
   return kPolicies[select_policy(m, n, k)].name;
 }
@@ -414,6 +417,27 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
     return xmk::check_launch("gemm");
   }
 
+  if (din == XMK_F32 && dout == XMK_F32 && xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) &&
+      xmk::aligned(out2, 16) && xmk::aligned(d->c, 16) && xmk::aligned(lhs.data, 4) && xmk::aligned(rhs.data, 4)) {
+    GemmParams p;
+    p.a = lhs.data; p.b = rhs.data; p.out = out.data; p.c = d->beta != 0.0f ? d->c : nullptr;
+    p.bias = wants_bias ? d->bias : nullptr;
+    p.M = (int)m; p.N = (int)n; p.K = (int)k;
+    p.lda = lhs.leading_dim_stride; p.ldb = rhs.leading_dim_stride; p.ldc = out.leading_dim_stride;
+    p.sa = lhs.batch_stride; p.sb = rhs.batch_stride; p.sc = out.batch_stride;
+    p.alpha = d->alpha; p.beta = d->beta; p.act = act;
+    p.out_alt[0] = out1; p.out_alt[1] = out2; p.sbias = 0;
+    if (qkv) { p.sa = 0; p.sc = 0; p.sbias = n; }
+    auto vec4 = [](const xmk_matrix& x) {
+      return (xmk::aligned(x.data, 16) && x.leading_dim_stride % 4 == 0 && x.batch_stride % 4 == 0 && x.num_cols % 4 == 0) ? 4 : 1;
+    };
+    p.vec_a = vec4(lhs);
+    p.vec_b = vec4(rhs);
+    xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d -> mfma_f32_128x128x16", (long long)m,
+               (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose, rhs.transpose);
+    launch_gemm_f32(p, lhs.transpose != 0, rhs.transpose == 0, qkv ? 3 : (int)d->batch_size, st);
+    return xmk::check_launch("gemm");
+  }
   if (din == XMK_S8 && (d->alpha != 1.0f || d->beta != 0.0f || d->epilogue != XMK_EPI_DEFAULT))
     return xmk::fail(XMK_UNIMPLEMENTED, "gemm: s8 x s8 -> s32 supports alpha=1, beta=0, no epilogue");
   GenericParams g;

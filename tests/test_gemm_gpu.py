@@ -140,7 +140,8 @@ def test_generic_path(xmk, oracle):
     bias = oracle.from_f32(oracle.normal((n,), 62), dt)
     _, ref = oracle.gemm(a, b, dt, dt, bias=bias, epilogue=oracle.EPI_BIAS_GELU)
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
-    assert xmk.gemm_policy_name(m, n, k, dtype_in=xmk.F32, dtype_out=xmk.F32) == "generic_64x64"
+    assert xmk.gemm_policy_name(m, n, k, dtype_in=xmk.F32, dtype_out=xmk.F32) == "mfma_f32_128x128x16"
+    assert xmk.gemm_policy_name(m, n, k, dtype_in=xmk.S8, dtype_out=xmk.S32) == "generic_64x64"
     xmk.run_gemm(to_dev(a, "bf16"), to_dev(b, "bf16"), out, bias=to_dev(bias, "bf16"),
                  epilogue=xmk.EPI_BIAS_GELU)
     torch.cuda.synchronize()
@@ -316,3 +317,40 @@ def test_gathered_operands_batched_f32_out(xmk, oracle):
     torch.cuda.synchronize()
     _, ref = oracle.gemm(a2, b2, dt, dt)
     _check(oracle, o2.float().cpu().numpy(), ref[0])
+
+
+@pytest.mark.parametrize("lhs_t,rhs_t,out_t", [(0, 0, 0), (0, 1, 0), (1, 0, 0), (1, 1, 0), (0, 0, 1)])
+@pytest.mark.parametrize("m,n,k", [(37, 50, 45), (256, 384, 512), (300, 515, 1027), (129, 64, 20)])
+def test_f32_gemm(xmk, oracle, lhs_t, rhs_t, out_t, m, n, k):
+    """fp32 x fp32 -> fp32 on the fp32 matrix cores, every layout, aligned and odd sizes, with bias + ReLU.
+    Against a float64 product: fp32 accumulation over K terms, so rtol 1e-4 on the tensor's scale."""
+    a = oracle.normal((k, m) if lhs_t else (m, k), 90, 0.3).astype(np.float32)
+    b = oracle.normal((n, k) if rhs_t else (k, n), 91, 0.3).astype(np.float32)
+    bias = oracle.normal((n,), 92).astype(np.float32)
+    A = a.T if lhs_t else a
+    B = b.T if rhs_t else b
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    use_bias = not out_t
+    if use_bias:
+        ref = np.maximum(ref + bias.astype(np.float64), 0.0)
+    out = torch.full((n, m) if out_t else (m, n), float("nan"), dtype=torch.float32, device="cuda")
+    xmk.run_gemm(to_dev(a, "f32"), to_dev(b, "f32"), out, lhs_transpose=lhs_t, rhs_transpose=rhs_t,
+                 out_transpose=out_t, bias=to_dev(bias, "f32") if use_bias else None,
+                 epilogue=xmk.EPI_BIAS_RELU if use_bias else xmk.EPI_DEFAULT)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.float64)
+    got = got.T if out_t else got
+    assert np.abs(got - ref).max() <= 1e-4 * max(np.abs(ref).max(), 1.0), np.abs(got - ref).max()
+
+
+def test_f32_gemm_batched_beta(xmk, oracle):
+    """Batched fp32 product accumulated in place (beta = 1, alpha = 0.5)."""
+    bsz, m, n, k = 3, 130, 70, 96
+    a = oracle.normal((bsz, m, k), 93, 0.3).astype(np.float32)
+    b = oracle.normal((bsz, k, n), 94, 0.3).astype(np.float32)
+    c = oracle.normal((bsz, m, n), 95).astype(np.float32)
+    out = to_dev(c, "f32").clone()
+    xmk.run_gemm(to_dev(a, "f32"), to_dev(b, "f32"), out, c=out, alpha=0.5, beta=1.0)
+    torch.cuda.synchronize()
+    ref = 0.5 * (a.astype(np.float64) @ b.astype(np.float64)) + c
+    assert np.abs(out.cpu().numpy() - ref).max() <= 1e-4 * np.abs(ref).max()
