@@ -17,11 +17,13 @@
 // holding four consecutive output columns of one row.
 //
 // 16-bit operands whose strides or sizes the direct loads cannot take run the same kernel with a
-// gathering loader, fp32 operands the fp32 MFMA kernel (gemm_f32.hip); what is left (int8, outputs
-// that are not 16-byte aligned) runs gemm_generic_kernel, a plain LDS-tiled kernel.  This is where
+// gathering loader, fp32 operands the fp32 MFMA kernel (gemm_f32.hip), int8 operands the int8 MFMA
+// kernel (gemm_s8.hip); what is left (outputs that are not 16-byte aligned) runs
+// gemm_generic_kernel, a plain LDS-tiled kernel.  This is where
 // the reference falls back to oneDNN (onednn_matmul_utils.cc:394-491).
 #include "gemm_f32.h"
 #include "gemm_kernel.h"
+#include "gemm_s8.h"
 
 namespace {
 
@@ -194,6 +196,7 @@ extern "C" const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int
   (void)rhs_transpose;
   const bool sixteen = dtype_in == XMK_BF16 || dtype_in == XMK_F16;
   if (dtype_in == XMK_F32 && dtype_out == XMK_F32) return "mfma_f32_128x128x16";
+  if (dtype_in == XMK_S8 && dtype_out == XMK_S32) return "mfma_s8_128x128x64";
   if (!sixteen || !(dtype_out == dtype_in || dtype_out == XMK_F32)) return "generic_64x64";
   return kPolicies[select_policy(m, n, k)].name;
 }
@@ -440,6 +443,24 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
   }
   if (din == XMK_S8 && (d->alpha != 1.0f || d->beta != 0.0f || d->epilogue != XMK_EPI_DEFAULT))
     return xmk::fail(XMK_UNIMPLEMENTED, "gemm: s8 x s8 -> s32 supports alpha=1, beta=0, no epilogue");
+  if (din == XMK_S8 && dout == XMK_S32 && xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) && xmk::aligned(out2, 16)) {
+    GemmParams p{};
+    p.a = lhs.data; p.b = rhs.data; p.out = out.data;
+    p.M = (int)m; p.N = (int)n; p.K = (int)k;
+    p.lda = lhs.leading_dim_stride; p.ldb = rhs.leading_dim_stride; p.ldc = out.leading_dim_stride;
+    p.sa = lhs.batch_stride; p.sb = rhs.batch_stride; p.sc = out.batch_stride;
+    p.out_alt[0] = out1; p.out_alt[1] = out2;
+    if (qkv) { p.sa = 0; p.sc = 0; }
+    auto vec16 = [](const xmk_matrix& x) {
+      return (xmk::aligned(x.data, 16) && x.leading_dim_stride % 16 == 0 && x.batch_stride % 16 == 0 && x.num_cols % 16 == 0) ? 16 : 1;
+    };
+    p.vec_a = vec16(lhs);
+    p.vec_b = vec16(rhs);
+    xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d -> mfma_s8_128x128x64", (long long)m,
+               (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose, rhs.transpose);
+    launch_gemm_s8(p, lhs.transpose != 0, rhs.transpose == 0, qkv ? 3 : (int)d->batch_size, st);
+    return xmk::check_launch("gemm");
+  }
   GenericParams g;
   g.a = lhs.data; g.b = rhs.data; g.out = out.data; g.c = d->beta != 0.0f ? d->c : nullptr;
   g.bias = wants_bias ? d->bias : nullptr;

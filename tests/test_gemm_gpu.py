@@ -141,7 +141,7 @@ def test_generic_path(xmk, oracle):
     _, ref = oracle.gemm(a, b, dt, dt, bias=bias, epilogue=oracle.EPI_BIAS_GELU)
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     assert xmk.gemm_policy_name(m, n, k, dtype_in=xmk.F32, dtype_out=xmk.F32) == "mfma_f32_128x128x16"
-    assert xmk.gemm_policy_name(m, n, k, dtype_in=xmk.S8, dtype_out=xmk.S32) == "generic_64x64"
+    assert xmk.gemm_policy_name(m, n, k, dtype_in=xmk.S8, dtype_out=xmk.S32) == "mfma_s8_128x128x64"
     xmk.run_gemm(to_dev(a, "bf16"), to_dev(b, "bf16"), out, bias=to_dev(bias, "bf16"),
                  epilogue=xmk.EPI_BIAS_GELU)
     torch.cuda.synchronize()
@@ -354,3 +354,31 @@ def test_f32_gemm_batched_beta(xmk, oracle):
     torch.cuda.synchronize()
     ref = 0.5 * (a.astype(np.float64) @ b.astype(np.float64)) + c
     assert np.abs(out.cpu().numpy() - ref).max() <= 1e-4 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("lhs_t,rhs_t,out_t", [(0, 0, 0), (0, 1, 0), (1, 0, 0), (1, 1, 0), (0, 1, 1)])
+@pytest.mark.parametrize("m,n,k", [(37, 50, 45), (256, 384, 512), (300, 515, 1027), (129, 64, 20)])
+def test_s8_gemm_is_bit_exact(xmk, lhs_t, rhs_t, out_t, m, n, k):
+    """s8 x s8 -> s32 on the int8 matrix cores: integer arithmetic, so bit exact against an int64 product,
+    in every layout, for aligned and odd sizes; and a batched product."""
+    g = torch.Generator(device="cpu").manual_seed(m * 131 + n * 7 + k)
+    a = torch.randint(-128, 128, (k, m) if lhs_t else (m, k), dtype=torch.int8, generator=g)
+    b = torch.randint(-128, 128, (n, k) if rhs_t else (k, n), dtype=torch.int8, generator=g)
+    A = (a.T if lhs_t else a).to(torch.int64)
+    B = (b.T if rhs_t else b).to(torch.int64)
+    ref = (A @ B).to(torch.int32)
+    out = torch.full((n, m) if out_t else (m, n), -7, dtype=torch.int32, device="cuda")
+    xmk.run_gemm(a.cuda(), b.cuda(), out, lhs_transpose=lhs_t, rhs_transpose=rhs_t, out_transpose=out_t)
+    torch.cuda.synchronize()
+    got = out.cpu()
+    assert torch.equal(got.T if out_t else got, ref)
+
+
+def test_s8_gemm_batched(xmk):
+    g = torch.Generator(device="cpu").manual_seed(5)
+    a = torch.randint(-128, 128, (3, 70, 96), dtype=torch.int8, generator=g)
+    b = torch.randint(-128, 128, (3, 96, 130), dtype=torch.int8, generator=g)
+    out = torch.empty((3, 70, 130), dtype=torch.int32, device="cuda")
+    xmk.run_gemm(a.cuda(), b.cuda(), out)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), torch.bmm(a.to(torch.int64), b.to(torch.int64)).to(torch.int32))
