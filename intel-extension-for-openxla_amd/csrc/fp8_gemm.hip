@@ -11,6 +11,7 @@
 // B stored [K,N] (rhs_transpose == 0) runs a plain tiled kernel.
 #include <utility>
 
+#include "gemm_gather8.h"
 #include "gemm_kernel.h"
 
 namespace {
@@ -213,7 +214,137 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
   });
 }
 
-// Plain tiled kernel for any layout / size: 64x64 tile, fp8 decoded with the hardware
+// Any layout, size and alignment on the matrix cores: the operands are gathered (gemm_gather8.h) into
+// the k-contiguous LDS layout, 16-byte chunks of 16 k; a lane's two neighbouring chunks are one operand
+// of v_mfma_scale_f32_32x32x64_f8f6f4 (row l % 32, k = 32 (l / 32) .. +31).  256 threads = 4 waves in
+// 2 x 2, tile 64 TW x 64 TW x 64, 4 LDS stages; the structure of the int8 kernel (gemm_s8.hip).
+template <int TW, int NSTAGE, int AMODE, int BMODE>
+__global__ __launch_bounds__(256) void fp8_gemm_gather_kernel(Fp8Params p) {
+  using namespace gather8;
+  constexpr bool b_kc = BMODE != MC;
+  constexpr int BM = 64 * TW, BN = 64 * TW;
+  constexpr int OP_BYTES = BM * BKB;
+  constexpr int STAGE = 2 * OP_BYTES;
+  constexpr int NLD = OP_BYTES / (256 * 16);
+  __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x % p.tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int8_t* A = reinterpret_cast<const int8_t*>(p.a);
+  const int8_t* B = reinterpret_cast<const int8_t*>(p.b);
+  const int8_t* a_tile = A + (int64_t)m0 * p.K;                       // A is [M, K]
+  const int8_t* b_tile = b_kc ? B + (int64_t)n0 * p.K : B + n0;       // B is [N, K] or [K, N]
+  const int64_t ldb = b_kc ? p.K : p.N;
+  const int64_t b_step = b_kc ? BKB : (int64_t)BKB * p.N;
+
+  floatx16 acc[TW][TW];
+#pragma unroll
+  for (int i = 0; i < TW; ++i)
+#pragma unroll
+    for (int j = 0; j < TW; ++j) acc[i][j] = zero16();
+
+  const int KT = (p.K + BKB - 1) / BKB;
+  auto load_step = [&](int kt, intx4 (&ga)[NLD], intx4 (&gb)[NLD]) {
+    const int kleft = p.K - kt * BKB;  // <= 0 past the end: zeros (fp8 zero is the zero byte)
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      ga[i] = gather<AMODE>(a_tile, A, p.K, p.M - m0, kleft, i, tid);
+      gb[i] = gather<BMODE>(b_tile, B, ldb, p.N - n0, kleft, i, tid);
+    }
+    a_tile += BKB;
+    b_tile += b_step;
+  };
+  auto store_step = [&](char* stage, const intx4 (&ga)[NLD], const intx4 (&gb)[NLD]) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      *reinterpret_cast<intx4*>(stage + i * 4096 + tid * 16) = ga[i];
+      *reinterpret_cast<intx4*>(stage + OP_BYTES + i * 4096 + tid * 16) = gb[i];
+    }
+  };
+  Fp8Frag fa_addr, fb_addr;
+  fa_addr.init(wm * 32 * TW, lane);
+  fb_addr.init(wn * 32 * TW, lane);
+
+  {
+    intx4 ga[NLD], gb[NLD];
+    for (int st = 0; st < NSTAGE - 1; ++st) {
+      load_step(st, ga, gb);
+      store_step(lds + st * STAGE, ga, gb);
+    }
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const char* cur = lds + (kt % NSTAGE) * STAGE;
+    char* wr = lds + ((kt + NSTAGE - 1) % NSTAGE) * STAGE;  // read during step kt - 1
+    intx4 ga[NLD], gb[NLD];
+    load_step(kt + NSTAGE - 1, ga, gb);
+    intx8 fa[TW], fb[TW];
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+      fa[t] = fa_addr.read(cur, t);
+      fb[t] = fb_addr.read(cur + OP_BYTES, t);
+    }
+#pragma unroll
+    for (int ti = 0; ti < TW; ++ti)
+#pragma unroll
+      for (int tj = 0; tj < TW; ++tj) acc[ti][tj] = mfma_fp8(fb[tj], fa[ti], acc[ti][tj]);
+    store_step(wr, ga, gb);
+    __syncthreads();  // step kt + NSTAGE - 1 is in LDS for every wave; every wave is done with `cur`
+  }
+
+  // acc[i][j][e] is out[m][n], m = m0 + 32 TW wm + 32 i + lane % 32, n = n0 + 32 TW wn + 32 j + 8 (e/4) + 4 (lane/32) + e%4.
+  gemm_impl::GemmParams q{};
+  q.out = p.out;
+  q.M = p.M;
+  q.N = p.N;
+  q.ldc = p.N;
+  q.alpha = p.a_scale[0] * p.b_scale[0];
+  q.act = gemm_impl::ACT_NONE;
+#pragma unroll
+  for (int i = 0; i < TW; ++i) {
+    const int m = m0 + wm * 32 * TW + i * 32 + l32;
+#pragma unroll
+    for (int j = 0; j < TW; ++j) {
+      const floatx16 t = acc[i][j];
+      const int nb = n0 + wn * 32 * TW + j * 32 + g * 4;
+      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[0], t[1], t[2], t[3]}, m, nb, 0);
+      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[4], t[5], t[6], t[7]}, m, nb + 8, 0);
+      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[8], t[9], t[10], t[11]}, m, nb + 16, 0);
+      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[12], t[13], t[14], t[15]}, m, nb + 24, 0);
+    }
+  }
+}
+
+template <int TW, int AMODE>
+void launch_gather_b(const Fp8Params& p, int bmode, dim3 grid, hipStream_t st) {
+  using namespace gather8;
+  if (bmode == KC_VEC) hipLaunchKernelGGL((fp8_gemm_gather_kernel<TW, 4, AMODE, KC_VEC>), grid, dim3(256), 0, st, p);
+  else if (bmode == KC_SCALAR) hipLaunchKernelGGL((fp8_gemm_gather_kernel<TW, 4, AMODE, KC_SCALAR>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((fp8_gemm_gather_kernel<TW, 4, AMODE, MC>), grid, dim3(256), 0, st, p);
+}
+
+// a_vec / b_vec: 16-byte aligned pointer and K % 16 == 0 (the k-contiguous operand can be read 16 bytes at a time).
+void launch_gather(Fp8Params& p, bool rhs_is_nk, bool a_vec, bool b_vec, hipStream_t st) {
+  using namespace gather8;
+  const bool large = xmk::ceil_div(p.M, 128) * xmk::ceil_div(p.N, 128) >= 256;
+  const int edge = large ? 128 : 64;
+  p.tiles_m = (int)xmk::ceil_div(p.M, edge);
+  p.tiles_n = (int)xmk::ceil_div(p.N, edge);
+  const dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+  const int bmode = !rhs_is_nk ? MC : (b_vec ? KC_VEC : KC_SCALAR);
+  if (large) {
+    if (a_vec) launch_gather_b<2, KC_VEC>(p, bmode, grid, st);
+    else launch_gather_b<2, KC_SCALAR>(p, bmode, grid, st);
+  } else {
+    if (a_vec) launch_gather_b<1, KC_VEC>(p, bmode, grid, st);
+    else launch_gather_b<1, KC_SCALAR>(p, bmode, grid, st);
+  }
+}
+
+// Plain tiled kernel for outputs that are not 8-byte aligned: 64x64 tile, fp8 decoded with the hardware
 // conversion while staging, fp32 FMA.
 __global__ __launch_bounds__(256) void fp8_gemm_generic_kernel(Fp8Params p, int rhs_transpose) {
   __shared__ float As[16][65];
@@ -283,6 +414,10 @@ extern "C" int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, 
       p.tiles_m = (int)xmk::ceil_div(m, 128); p.tiles_n = (int)xmk::ceil_div(n, 128);
       hipLaunchKernelGGL((fp8_gemm_kernel<128, 128, 2, 2, 4>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
     }
+  } else if (xmk::aligned(out, 8) && (int64_t)m * k < (int64_t)1 << 40) {
+    xmk::trace("fp8_gemm m=%lld n=%lld k=%lld rhs_t=%d -> mfma_gather", (long long)m, (long long)n, (long long)k,
+               rhs_transpose);
+    launch_gather(p, rhs_transpose != 0, k % 16 == 0 && xmk::aligned(a, 16), k % 16 == 0 && xmk::aligned(b, 16), st);
   } else {
     xmk::trace("fp8_gemm m=%lld n=%lld k=%lld rhs_t=%d -> generic_64x64", (long long)m, (long long)n,
                (long long)k, rhs_transpose);

@@ -11,46 +11,14 @@
 // a lane holds four consecutive output columns and stores them with one 16-byte store.
 #include "gemm_s8.h"
 
+#include "gemm_gather8.h"
+
 namespace gemm_impl {
 namespace {
 
-typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BKB = 64;  // k per K step = bytes of one LDS row
-enum : int { KC_VEC = 0, KC_SCALAR = 1, MC = 2 };
-
-__device__ __forceinline__ int swz4(int row) { return (row >> 2) & 3; }
-
-template <int MODE>
-__device__ __forceinline__ intx4 gather(const int8_t* base, const int8_t* safe, int64_t ld, int valid, int kleft, int i,
-                                        int tid) {
-  const int row = i * 64 + (tid >> 2);
-  const int k = ((tid & 3) ^ swz4(row)) * 16;
-  const bool in = row < valid;
-  intx4 v;
-  if constexpr (MODE == KC_VEC) {  // K % 16 == 0: the chunk is inside the row or outside as a whole
-    const bool ok = in && k < kleft;
-    v = *reinterpret_cast<const intx4*>(ok ? base + (int64_t)row * ld + k : safe);
-    if (!ok) v = intx4{0, 0, 0, 0};
-  } else {
-    const int8_t* src = MODE == KC_SCALAR ? base + (int64_t)row * ld + k : base + (int64_t)k * ld + row;
-    const int64_t step = MODE == KC_SCALAR ? 1 : ld;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      uint32_t word = 0;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int j = 4 * w + b;
-        const bool ok = in && k + j < kleft;
-        const uint32_t x = (uint8_t) * (ok ? src + j * step : safe);
-        word |= (ok ? x : 0u) << (8 * b);
-      }
-      v[w] = (int)word;
-    }
-  }
-  return v;
-}
+using namespace gather8;
 
 template <int TW, int NSTAGE, int AMODE, int BMODE>
 __global__ __launch_bounds__(256) void gemm_s8_kernel(GemmParams p) {

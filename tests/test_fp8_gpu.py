@@ -19,6 +19,8 @@ def _quant(oracle, shape, seed):
     (256, 256, 128, True), (512, 384, 1024, True), (300, 260, 208, True), (64, 8, 16, True),
     (4136, 4104, 208, True),  # ragged edges of the 256x256 tile (taken when there are >= 256 tiles)
     (130, 72, 80, False), (256, 256, 256, False),
+    # the gathering kernel: [k,n]-stored B, K that is not a multiple of 16, odd N, both tile sizes
+    (300, 515, 1027, False), (37, 52, 45, True), (2100, 2060, 200, False), (2100, 2060, 72, True),
 ])
 def test_fp8_gemm_shapes(xmk, oracle, m, n, k, rhs_t):
     a, sa = _quant(oracle, (m, k), 1)
