@@ -207,6 +207,16 @@ int xmk_int4_gemm(const void* act, const void* qweight, const void* scales, cons
                   const void* bias, void* out, int64_t m, int64_t k, int64_t n,
                   int64_t group, void* stream);
 
+/* xmk_int4_gemm for many rows (prompt processing) with caller-provided scratch: when
+ * xmk_int4_gemm_workspace_bytes(m, k, n) is not 0 and the workspace (16-byte aligned) holds that many
+ * bytes, W = xmk_int4_dequant(...) is written to it once and out = fp16(act . W + bias) runs on the dense
+ * fp16 GEMM, so w IS rounded to fp16 on this path (a relative 2^-11 per weight, inside the tolerance of
+ * the direct kernel).  Otherwise the call is xmk_int4_gemm.  Not in the reference snapshot. */
+size_t xmk_int4_gemm_workspace_bytes(int64_t m, int64_t k, int64_t n);
+int xmk_int4_gemm_ws(const void* act, const void* qweight, const void* scales, const void* zeros,
+                     const void* bias, void* out, int64_t m, int64_t k, int64_t n, int64_t group,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
 /* The dequantised weight matrix itself, fp16 [K, N]: the bit-exact check
  * surface for the formula above. */
 int xmk_int4_dequant(const void* qweight, const void* scales, const void* zeros, void* w_out,

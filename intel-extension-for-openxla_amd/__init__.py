@@ -67,7 +67,8 @@ def lib():
                               ("xmk_gemm_policy_name", ctypes.c_char_p),
                               ("xmk_fmha_decode_workspace_bytes", ctypes.c_size_t),
                               ("xmk_fmha_bwd_workspace_bytes", ctypes.c_size_t),
-                              ("xmk_gemm_workspace_bytes", ctypes.c_size_t)):
+                              ("xmk_gemm_workspace_bytes", ctypes.c_size_t),
+                              ("xmk_int4_gemm_workspace_bytes", ctypes.c_size_t)):
             if hasattr(L, name):
                 getattr(L, name).restype = restype
         _lib = L
@@ -213,6 +214,22 @@ def int4_gemm(act, qweight, scales, zeros, out, *, group=128, bias=None, stream=
     _check(lib().xmk_int4_gemm(_ptr(act), _ptr(qweight), _ptr(scales), _ptr(zeros), _ptr(bias),
                                _ptr(out), ctypes.c_int64(m), ctypes.c_int64(k), ctypes.c_int64(n),
                                ctypes.c_int64(group), _stream(stream)))
+    return out
+
+
+def int4_gemm_workspace_bytes(m, k, n):
+    return lib().xmk_int4_gemm_workspace_bytes(ctypes.c_int64(m), ctypes.c_int64(k), ctypes.c_int64(n))
+
+
+def int4_gemm_ws(act, qweight, scales, zeros, out, workspace, *, group=128, bias=None, stream=None):
+    """xmk_int4_gemm_ws: with enough scratch and rows, dequantise once and run the dense fp16 GEMM."""
+    m, k = act.shape
+    n = qweight.shape[1]
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(lib().xmk_int4_gemm_ws(_ptr(act), _ptr(qweight), _ptr(scales), _ptr(zeros), _ptr(bias),
+                                  _ptr(out), ctypes.c_int64(m), ctypes.c_int64(k), ctypes.c_int64(n),
+                                  ctypes.c_int64(group), _ptr(workspace), ctypes.c_size_t(nbytes),
+                                  _stream(stream)))
     return out
 
 

@@ -170,6 +170,41 @@ void destroy_error(const XLA_FFI_Api* api, XLA_FFI_Error* e) {
   api->XLA_FFI_Error_Destroy(&a);
 }
 
+// Runs body(workspace) with `need` bytes of the executor's scratch when the API table has the allocator
+// entries and the allocation succeeds, else body(nullptr).  The scratch is handed back right after the
+// work is enqueued: the executor's allocator frees in stream order, so later work on the stream may reuse it.
+template <typename Body>
+int with_scratch(XLA_FFI_CallFrame* f, size_t need, Body&& body) {
+  const XLA_FFI_Api* api = f->api;
+  const bool can_allocate = need > 0 && api &&
+                            api->struct_size >= offsetof(XLA_FFI_Api, XLA_FFI_DeviceMemory_Free) + sizeof(void*) &&
+                            api->XLA_FFI_DeviceMemory_Allocate && api->XLA_FFI_DeviceMemory_Free;
+  if (can_allocate) {
+    XLA_FFI_DeviceMemory_Allocate_Args al;
+    al.struct_size = sizeof(al);
+    al.extension_start = nullptr;
+    al.ctx = f->ctx;
+    al.size = need;
+    al.alignment = 256;
+    al.data = nullptr;
+    XLA_FFI_Error* e = api->XLA_FFI_DeviceMemory_Allocate(&al);
+    if (!e && al.data) {
+      const int rc = body(al.data);
+      XLA_FFI_DeviceMemory_Free_Args fa;
+      fa.struct_size = sizeof(fa);
+      fa.extension_start = nullptr;
+      fa.ctx = f->ctx;
+      fa.size = need;
+      fa.data = al.data;
+      XLA_FFI_Error* fe = api->XLA_FFI_DeviceMemory_Free(&fa);
+      if (fe) destroy_error(api, fe);
+      return rc;
+    }
+    if (e) destroy_error(api, e);
+  }
+  return body(nullptr);
+}
+
 XLA_FFI_Error* gemm_common(XLA_FFI_CallFrame* f, bool lt) {
   if (metadata_query(f) || f->stage != XLA_FFI_ExecutionStage_EXECUTE) return nullptr;
   Frame fr{f};
@@ -207,35 +242,9 @@ XLA_FFI_Error* gemm_common(XLA_FFI_CallFrame* f, bool lt) {
   // Shapes that gain from a K split take their fp32 partial sums from the executor's scratch allocator
   // (the reference's handlers hold one too, sycl_custom_call.cc:154-156), when the API table has it.
   const size_t need = xmk_gemm_workspace_bytes(&d);
-  const XLA_FFI_Api* api = f->api;
-  const bool can_allocate = need > 0 && api &&
-                            api->struct_size >= offsetof(XLA_FFI_Api, XLA_FFI_DeviceMemory_Free) + sizeof(void*) &&
-                            api->XLA_FFI_DeviceMemory_Allocate && api->XLA_FFI_DeviceMemory_Free;
-  if (can_allocate) {
-    XLA_FFI_DeviceMemory_Allocate_Args al;
-    al.struct_size = sizeof(al);
-    al.extension_start = nullptr;
-    al.ctx = f->ctx;
-    al.size = need;
-    al.alignment = 256;
-    al.data = nullptr;
-    XLA_FFI_Error* e = api->XLA_FFI_DeviceMemory_Allocate(&al);
-    if (!e && al.data) {
-      const int rc = xmk_gemm_ws(&d, al.data, need, stream);
-      // Freed in stream order by the executor's allocator: later work on this stream may reuse it.
-      XLA_FFI_DeviceMemory_Free_Args fa;
-      fa.struct_size = sizeof(fa);
-      fa.extension_start = nullptr;
-      fa.ctx = f->ctx;
-      fa.size = need;
-      fa.data = al.data;
-      XLA_FFI_Error* fe = api->XLA_FFI_DeviceMemory_Free(&fa);
-      if (fe) destroy_error(api, fe);
-      return finish(fr, rc);
-    }
-    if (e) destroy_error(api, e);  // no scratch: the unsplit kernel needs none
-  }
-  return finish(fr, xmk_gemm(&d, stream));
+  return finish(fr, with_scratch(f, need, [&](void* ws) {
+    return ws ? xmk_gemm_ws(&d, ws, need, stream) : xmk_gemm(&d, stream);  // no scratch: the unsplit kernel
+  }));
 }
 
 XLA_FFI_Error* fmha_common(XLA_FFI_CallFrame* f, bool with_bias) {
@@ -319,8 +328,12 @@ extern "C" XLA_FFI_Error* xmk_ffi_int4_gemm(XLA_FFI_CallFrame* f) {
     fr.fail(XMK_INVALID_ARGUMENT, "int4_gemm: operand shapes do not agree");
   void* stream = fr.stream();
   if (fr.code != XMK_OK) return finish(fr, XMK_OK);
-  return finish(fr, xmk_int4_gemm(act->data, qw->data, sc->data, zp->data, bias ? bias->data : nullptr, out->data, M,
-                                  K, N, K / groups, stream));
+  // Many rows (prompt processing): the dequantised weights go to executor scratch and the dense GEMM runs.
+  const size_t need = xmk_int4_gemm_workspace_bytes(M, K, N);
+  return finish(fr, with_scratch(f, need, [&](void* ws) {
+    return xmk_int4_gemm_ws(act->data, qw->data, sc->data, zp->data, bias ? bias->data : nullptr, out->data, M, K, N,
+                            K / groups, ws, ws ? need : 0, stream);
+  }));
 }
 
 extern "C" XLA_FFI_Error* xmk_ffi_cublas_lt_matmul_f8(XLA_FFI_CallFrame* f) {

@@ -154,6 +154,34 @@ def test_int4_handler(ffi, oracle):
     assert g <= 1e-2 and e <= 1e-2, (g, e)
 
 
+def test_int4_handler_takes_scratch_for_many_rows(ffi, oracle):
+    """256 rows: the handler asks the executor for K*N fp16 of scratch (dequantise once + dense GEMM) when the
+    API table has an allocator, and streams the packed weights when it has none."""
+    m, k, n, group = 256, 512, 256, 128
+    act = oracle.from_f32(oracle.normal((m, k), 60, 1.0), oracle.F16)
+    qw = oracle.words((k // 8, n), 61)
+    sc = oracle.from_f32(oracle.uniform((k // group, n), 62, 0.001, 0.02), oracle.F16)
+    zp = oracle.from_f32(oracle.uniform((k // group, n), 63, 0.0, 15.0), oracle.F16)
+    _, ref = oracle.int4_gemm(act, qw, sc, zp, group)
+    dact, dqw, dsc, dzp = to_dev(act, "f16"), to_dev(qw, "u32"), to_dev(sc, "f16"), to_dev(zp, "f16")
+
+    def allocator(size, alignment):
+        t = torch.empty((size + alignment,), dtype=torch.uint8, device="cuda")
+        return (t.data_ptr() + alignment - 1) // alignment * alignment, t
+
+    for alloc in (allocator, None):
+        out = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+        host = F.FakeHost(stream=torch.cuda.current_stream().cuda_stream, allocator=alloc)
+        f = host.frame([_buf(dact, F.F16), _buf(dqw, F.S32), _buf(dsc, F.F16), _buf(dzp, F.F16)], [_buf(out, F.F16)], {})
+        _ok(host, ffi.xmk_ffi_int4_gemm(C.byref(f)))
+        if alloc:
+            assert host.allocations == [(k * n * 2, 256)] and host.freed == [k * n * 2]
+        else:
+            assert host.allocations == []
+        g, e = oracle.rel_err(out.float().cpu().numpy(), ref)
+        assert g <= 1e-2 and e <= 1e-2, (alloc is not None, g, e)
+
+
 def test_f8_matmul_handler(ffi, oracle):
     m, n, k = 320, 264, 208
     a, sa = oracle.fp8_quantize(oracle.normal((m, k), 50))

@@ -83,6 +83,33 @@ def test_int4_gemm_linearity_full_size(xmk, oracle):
     assert err < 1e-2
 
 
+@pytest.mark.parametrize("m,k,n,group,with_bias", [(256, 512, 1024, 128, True), (200, 1024, 328, 64, False)])
+def test_int4_gemm_many_rows_with_scratch(xmk, oracle, m, k, n, group, with_bias):
+    """Prompt-sized row counts: with the scratch xmk_int4_gemm_workspace_bytes asks for, the weights are
+    dequantised once and the dense fp16 GEMM runs; without it the streaming kernel runs.  Both within
+    1e-2 of the fp32 recompute, and of the recompute from fp16-rounded weights."""
+    act, qw, s, z = _case(oracle, m, k, n, group, 2000 + m)
+    bias = oracle.from_f32(oracle.normal((n,), 56), oracle.F16) if with_bias else None
+    _, ref = oracle.int4_gemm(act, qw, s, z, group, bias=bias)
+    _, ref16 = oracle.int4_gemm(act, qw, s, z, group, bias=bias, round_weights=True)
+    need = xmk.int4_gemm_workspace_bytes(m, k, n)
+    assert need == k * n * 2
+    assert xmk.int4_gemm_workspace_bytes(32, k, n) == 0   # decode-sized calls never ask for scratch
+    ws = torch.empty((need,), dtype=torch.uint8, device="cuda")
+    dev = [to_dev(act, "f16"), to_dev(qw, "u32"), to_dev(s, "f16"), to_dev(z, "f16")]
+    dbias = None if bias is None else to_dev(bias, "f16")
+    outs = []
+    for scratch in (ws, None):
+        out = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
+        xmk.int4_gemm_ws(*dev, out, scratch, group=group, bias=dbias)
+        torch.cuda.synchronize()
+        for r in (ref, ref16):
+            g, e = oracle.rel_err(out.float().cpu().numpy(), r)
+            assert g <= 1e-2 and e <= 1e-2, (scratch is not None, g, e)
+        outs.append(out.float())
+    assert (outs[0] - outs[1]).abs().max().item() <= 1e-2 * outs[1].abs().max().item()
+
+
 def test_int4_errors(xmk):
     a = torch.zeros((1, 256), dtype=torch.float16, device="cuda")
     qw = torch.zeros((32, 64), dtype=torch.int32, device="cuda")
@@ -93,4 +120,11 @@ def test_int4_errors(xmk):
     assert e.value.code == xmk.INVALID_ARGUMENT
     with pytest.raises(xmk.XmkError) as e:
         xmk.int4_gemm(a, qw, sz, sz, out, group=8)
+    assert e.value.code == xmk.UNIMPLEMENTED
+    # the same contract on the dense path
+    a2 = torch.zeros((256, 256), dtype=torch.float16, device="cuda")
+    out2 = torch.zeros((256, 64), dtype=torch.float16, device="cuda")
+    ws = torch.empty((xmk.int4_gemm_workspace_bytes(256, 256, 64),), dtype=torch.uint8, device="cuda")
+    with pytest.raises(xmk.XmkError) as e:
+        xmk.int4_gemm_ws(a2, qw, sz, sz, out2, ws, group=8)
     assert e.value.code == xmk.UNIMPLEMENTED
