@@ -112,6 +112,9 @@ __device__ __forceinline__ float half_at(const Words<NWORDS>& r, int c) {
 // SPG  : 32-channel k-steps per quantisation group (group = 32*SPG)
 // NW   : waves per block; wave w takes groups w, w+NW, ... and the partial
 //        sums meet in LDS in a fixed order (deterministic result)
+// SPREAD: 2 to 4 rows (RI = 1) or 5 to 8 rows (RI = 2): activation row r is fed to the MFMA as row
+//        (4 / RI) r, the rows between are zeros, so that the live rows come out in accumulator elements
+//        0 (and 2) of every lane group and the per-group fix-up touches RI elements per lane instead of four
 // SK   : K is also split over gridDim.y work-groups; slice y writes its fp32 partial sums
 //        [32 rows][N] to partial + y * 32 * N and applies no epilogue (the consumer adds the
 //        slices in a fixed order)
@@ -131,7 +134,7 @@ struct Int4Problem {
   float* partial;
 };
 
-template <int W, int MT, int RI, int SPG, int NW, bool SK>
+template <int W, int MT, int RI, int SPG, int NW, bool SK, bool SPREAD>
 __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0) {
   const bool second = (int)blockIdx.x >= blocks0;
   const int bx = (int)blockIdx.x - (second ? blocks0 : 0);
@@ -146,7 +149,9 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   const xmk::Int4Epilogue ep = second ? p1.ep : p0.ep;
   float* __restrict__ partial = second ? p1.partial : p0.partial;
   constexpr int NCOL = 16 * W;
-  constexpr int ROWS = MT == 2 ? 32 : (RI == 4 ? 16 : RI);  // rows the block reduces
+  static_assert(!SPREAD || (MT == 1 && (RI == 1 || RI == 2)), "spread rows: one tile, one or two live elements per lane");
+  constexpr int ROWS = SPREAD ? 4 * RI : (MT == 2 ? 32 : (RI == 4 ? 16 : RI));  // rows the block reduces
+  constexpr int ESTEP = SPREAD ? 4 / RI : 1;  // live accumulator elements are 0, ESTEP, ...
   __shared__ float red[NW][ROWS][NCOL];
 
   const int lane = threadIdx.x & 63;
@@ -168,8 +173,9 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   uint32_t voff_a[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + col16;
-    voff_a[mt] = (m_base + m < M) ? (uint32_t)((m * K + 8 * kg) * 2) : kOob;
+    const int m = SPREAD ? col16 / ESTEP : mt * 16 + col16;
+    const bool fed = !SPREAD || col16 % ESTEP == 0;  // MFMA rows ESTEP r carry activation row r, the others zeros
+    voff_a[mt] = (fed && m_base + m < M) ? (uint32_t)((m * K + 8 * kg) * 2) : kOob;
   }
 
   floatx4 acc[MT][W];
@@ -243,8 +249,10 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int i = 0; i < RI; ++i)
-          acc[mt][c][i] = fmaf(sc, d[mt][c][i] - fmaf(z, asum[mt][i], aoff[mt][i]), acc[mt][c][i]);
+        for (int i = 0; i < RI; ++i) {
+          const int e = i * ESTEP;
+          acc[mt][c][e] = fmaf(sc, d[mt][c][e] - fmaf(z, asum[mt][e], aoff[mt][e]), acc[mt][c][e]);
+        }
     }
   };
 
@@ -265,7 +273,12 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   }
 
   // Lane holds rows 4*kg+i (+16 mt) of columns col16*W+c.
-  if (RI == 4 || kg == 0) {
+  if constexpr (SPREAD) {
+#pragma unroll
+    for (int j = 0; j < RI; ++j)
+#pragma unroll
+      for (int c = 0; c < W; ++c) red[wave][kg * RI + j][col16 * W + c] = acc[0][c][j * ESTEP];
+  } else if (RI == 4 || kg == 0) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -370,29 +383,29 @@ struct Config {
   bool operator==(const Config& o) const { return w == o.w && nw == o.nw && ksplit == o.ksplit; }
 };
 
-template <int W, int MT, int RI, int SPG, int NW>
+template <int W, int MT, int RI, int SPG, int NW, bool SPREAD>
 void launch(const Int4Problem& a, const Int4Problem* b, int ksplit, hipStream_t st) {
   const int blocks0 = (int)xmk::ceil_div(a.N, 16 * W);
   const int blocks = blocks0 + (b ? (int)xmk::ceil_div(b->N, 16 * W) : 0);
   const Int4Problem& second = b ? *b : a;
   if (ksplit > 1) {
     if constexpr (W == 4 && MT == 1) {  // the only shape the split is planned for
-      hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true>), dim3(blocks, ksplit), dim3(NW * 64), 0, st, a,
+      hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true, SPREAD>), dim3(blocks, ksplit), dim3(NW * 64), 0, st, a,
                          second, blocks0);
       return;
     }
   }
-  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false>), dim3(blocks), dim3(NW * 64), 0, st, a, second,
+  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false, SPREAD>), dim3(blocks), dim3(NW * 64), 0, st, a, second,
                      blocks0);
 }
 
-template <int W, int MT, int RI, int NW>
+template <int W, int MT, int RI, int NW, bool SPREAD = false>
 int launch_spg(int spg, const Int4Problem& a, const Int4Problem* b, int ksplit, hipStream_t st) {
   switch (spg) {
-    case 1: launch<W, MT, RI, 1, NW>(a, b, ksplit, st); break;
-    case 2: launch<W, MT, RI, 2, NW>(a, b, ksplit, st); break;
-    case 4: launch<W, MT, RI, 4, NW>(a, b, ksplit, st); break;
-    case 8: launch<W, MT, RI, 8, NW>(a, b, ksplit, st); break;
+    case 1: launch<W, MT, RI, 1, NW, SPREAD>(a, b, ksplit, st); break;
+    case 2: launch<W, MT, RI, 2, NW, SPREAD>(a, b, ksplit, st); break;
+    case 4: launch<W, MT, RI, 4, NW, SPREAD>(a, b, ksplit, st); break;
+    case 8: launch<W, MT, RI, 8, NW, SPREAD>(a, b, ksplit, st); break;
     default: return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   }
   return XMK_OK;
@@ -467,6 +480,12 @@ int launch_cfg(const Config& cfg, int spg, const xmk::Int4Call& a, const xmk::In
 #define XMK_INT4_CASE(WW)                                                            \
   do {                                                                               \
     if (rows > 16) rc = launch_spg<WW, 2, 4, 8>(spg, pa, pb, cfg.ksplit, st);        \
+    else if (rows > 1 && rows <= 4)                                                  \
+      rc = cfg.nw == 4 ? launch_spg<WW, 1, 1, 4, true>(spg, pa, pb, cfg.ksplit, st)  \
+                       : launch_spg<WW, 1, 1, 8, true>(spg, pa, pb, cfg.ksplit, st); \
+    else if (rows > 4 && rows <= 8)                                                  \
+      rc = cfg.nw == 4 ? launch_spg<WW, 1, 2, 4, true>(spg, pa, pb, cfg.ksplit, st)  \
+                       : launch_spg<WW, 1, 2, 8, true>(spg, pa, pb, cfg.ksplit, st); \
     else if (rows > 1) rc = cfg.nw == 4 ? launch_spg<WW, 1, 4, 4>(spg, pa, pb, cfg.ksplit, st)   \
                                         : launch_spg<WW, 1, 4, 8>(spg, pa, pb, cfg.ksplit, st); \
     else rc = cfg.nw == 16 ? launch_spg<WW, 1, 1, 16>(spg, pa, pb, cfg.ksplit, st)   \

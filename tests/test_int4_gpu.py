@@ -52,6 +52,11 @@ def test_int4_gemm_gptj_mlp_shape(xmk, oracle, m):
     (17, 512, 200, 64, True),       # ragged N (not a multiple of the block's columns), two row tiles
     (33, 256, 72, 256, False),      # M > 32: second launch
     (16, 1024, 1024, 128, True),
+    (2, 512, 136, 128, True),       # 2-4 rows and 5-8 rows take the variants that feed the rows spread out
+    (6, 1024, 200, 64, False),
+    (7, 4096, 4096, 128, True),
+    (36, 256, 72, 32, True),        # 32 rows + 4 in a second launch
+    (40, 512, 264, 128, False),     # 32 rows + 8
 ])
 def test_int4_gemm_shapes(xmk, oracle, m, k, n, group, with_bias):
     act, qw, s, z = _case(oracle, m, k, n, group, 1000 + m + n)
