@@ -644,6 +644,7 @@ constexpr Policy kPolicies[] = {
     {"mfma_128x128x64_w2x2_s3", 128, 128, 2, 2, 64, 3},
     {"mfma_128x64x64_w2x2_s4", 128, 64, 2, 2, 64, 4},
     {"mfma_64x64x64_w2x2_s4", 64, 64, 2, 2, 64, 4},
+    {"mfma_256x128x64_w2x2_s3", 256, 128, 2, 2, 64, 3},
 };
 constexpr int kNumPolicies = sizeof(kPolicies) / sizeof(kPolicies[0]);
 
@@ -668,7 +669,7 @@ inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1) {
   // Heuristic: the policy with the best estimated throughput = (what the tile sustains when the
   // device is full) x (share of the 256 CUs busy over the tile waves) x (share of the tiles' area
   // inside the matrix).  The per-tile figures are measured large-shape rates relative to 256x256.
-  static constexpr float kTileRate[kNumPolicies] = {1.0f, 0.75f, 0.60f, 0.55f};
+  static constexpr float kTileRate[kNumPolicies] = {1.0f, 0.75f, 0.60f, 0.55f, 0.90f};
   int best = kNumPolicies - 1;
   float best_score = -1.0f;
   for (int i = 0; i < kNumPolicies; ++i) {
@@ -700,6 +701,7 @@ void launch_policy(int pol, GemmParams& p, int batch, hipStream_t st) {
     case 0: launch_mfma<T, OutF32, A_MC, B_MC, 256, 256, 2, 2, 32, 4>(p, batch, st); break;
     case 1: launch_mfma<T, OutF32, A_MC, B_MC, 128, 128, 2, 2, 64, 3>(p, batch, st); break;
     case 2: launch_mfma<T, OutF32, A_MC, B_MC, 128, 64, 2, 2, 64, 4>(p, batch, st); break;
+    case 4: launch_mfma<T, OutF32, A_MC, B_MC, 256, 128, 2, 2, 64, 3>(p, batch, st); break;
     default: launch_mfma<T, OutF32, A_MC, B_MC, 64, 64, 2, 2, 64, 4>(p, batch, st); break;
   }
 }

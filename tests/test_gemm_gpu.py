@@ -59,6 +59,27 @@ def test_layouts(xmk, oracle, dt_name, lhs_t, rhs_t, out_t, m, n, k):
     _check(oracle, got.T if out_t else got, ref[0])
 
 
+@pytest.mark.parametrize("dt_name", ["BF16", "F16"])
+@pytest.mark.parametrize("lhs_t,rhs_t", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k", [(2048, 4096, 200), (1800, 4000, 136)])
+def test_tile_256x128(xmk, oracle, dt_name, lhs_t, rhs_t, m, n, k):
+    """Shapes whose 256x128 tiles number about one per CU take that tile (K step 64, three stages):
+    every operand layout, a K tail, and tiles that hang over the last rows and columns."""
+    assert xmk.gemm_policy_name(m, n, k, rhs_transpose=bool(rhs_t)) == "mfma_256x128x64_w2x2_s3"
+    dt = getattr(oracle, dt_name)
+    kind = _kind(dt, oracle)
+    a = oracle.from_f32(oracle.normal((k, m) if lhs_t else (m, k), 12, 0.3), dt)
+    b = oracle.from_f32(oracle.normal((n, k) if rhs_t else (k, n), 13, 0.3), dt)
+    bias = oracle.from_f32(oracle.normal((n,), 14, 0.5), dt)
+    _, ref = oracle.gemm(a, b, dt, dt, lhs_t=lhs_t, rhs_t=rhs_t, bias=bias, epilogue=oracle.EPI_BIAS)
+    tdt = torch.bfloat16 if kind == "bf16" else torch.float16
+    out = torch.full((m, n), float("nan"), dtype=tdt, device="cuda")
+    xmk.run_gemm(to_dev(a, kind), to_dev(b, kind), out, lhs_transpose=lhs_t, rhs_transpose=rhs_t,
+                 bias=to_dev(bias, kind), epilogue=xmk.EPI_BIAS)
+    torch.cuda.synchronize()
+    _check(oracle, out.float().cpu().numpy(), ref[0])
+
+
 @pytest.mark.parametrize("epi", ["DEFAULT", "RELU", "GELU", "BIAS", "BIAS_RELU", "BIAS_GELU"])
 @pytest.mark.parametrize("beta", [0.0, 1.0, 0.5])
 def test_epilogues(xmk, oracle, epi, beta):
