@@ -135,9 +135,13 @@ struct Int4Problem {
 };
 
 template <int W, int MT, int RI, int SPG, int NW, bool SK, bool SPREAD>
-__global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0) {
-  const bool second = (int)blockIdx.x >= blocks0;
-  const int bx = (int)blockIdx.x - (second ? blocks0 : 0);
+__global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0, int mixed) {
+  // mixed (two K-split products of equal width): the products alternate from one block to the next, and
+  // the alternation flips between the first and the second half of the K slices, so that work-groups
+  // which are half a grid apart -- the ones that end up sharing a CU -- belong to different products
+  // and every CU gets the same share of the longer reduction.
+  const bool second = (SK && mixed) ? (((int)blockIdx.x + (int)(blockIdx.y >> 1)) & 1) != 0 : (int)blockIdx.x >= blocks0;
+  const int bx = (SK && mixed) ? (int)blockIdx.x >> 1 : (int)blockIdx.x - (second ? blocks0 : 0);
   const _Float16* __restrict__ act = second ? p1.act : p0.act;
   const uint32_t* __restrict__ qw = second ? p1.qw : p0.qw;
   const _Float16* __restrict__ scales = second ? p1.scales : p0.scales;
@@ -390,13 +394,14 @@ void launch(const Int4Problem& a, const Int4Problem* b, int ksplit, hipStream_t 
   const Int4Problem& second = b ? *b : a;
   if (ksplit > 1) {
     if constexpr (W == 4 && MT == 1) {  // the only shape the split is planned for
+      const int mixed = b && blocks == 2 * blocks0 && ksplit % 4 == 0 ? 1 : 0;
       hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true, SPREAD>), dim3(blocks, ksplit), dim3(NW * 64), 0, st, a,
-                         second, blocks0);
+                         second, blocks0, mixed);
       return;
     }
   }
   hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false, SPREAD>), dim3(blocks), dim3(NW * 64), 0, st, a, second,
-                     blocks0);
+                     blocks0, 0);
 }
 
 template <int W, int MT, int RI, int NW, bool SPREAD = false>
