@@ -125,8 +125,13 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS) ? 2 : 1) void fmha_bwd_ke
   // unit stream the same tiles.
   const int wg = (int)(blockIdx.x % 8) * p.per_xcd + (int)(blockIdx.x / 8);
   if (wg >= p.total) return;
-  const int unit = wg / p.nob;
-  const int ob = OWNER_K ? wg % p.nob : p.nob - 1 - wg % p.nob;  // causal: heaviest blocks first
+  // Inside the range, units go four at a time, owner blocks outermost and (causal) heaviest first, so that an
+  // XCD's slots run dry at about the same time.
+  constexpr int UG = 4;
+  const int ublk = wg / (UG * p.nob), r = wg % (UG * p.nob);
+  const int gb = min(UG, p.total / p.nob - ublk * UG);  // units in this group (the last may hold fewer)
+  const int unit = ublk * UG + r % gb;
+  const int ob = OWNER_K ? r / gb : p.nob - 1 - r / gb;
   const int o0 = ob * BO;
   const int H = p.H;
   const int n_own = OWNER_K ? p.T : p.F;   // owner rows of the unit
