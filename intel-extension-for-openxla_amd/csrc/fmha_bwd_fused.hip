@@ -17,6 +17,7 @@
 //             contraction runs over the streamed rows); the streamed tile is read with the LDS
 //             transpose loads.
 // The streamed tiles go from global memory straight into LDS, two stages.
+#include <algorithm>
 #include <utility>
 
 #include "common.h"
@@ -86,7 +87,7 @@ struct KParams {
   void* out2;         // P^T dO (dV), owner = keys only
   int H, F, T;
   int nob;            // owner blocks per unit
-  int total, per_xcd;
+  int total, per_xcd, ug;
   float scale;
 };
 
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS) ? 2 : 1) void fmha_bwd_ke
   if (wg >= p.total) return;
   // Inside the range, units go four at a time, owner blocks outermost and (causal) heaviest first, so that an
   // XCD's slots run dry at about the same time.
-  constexpr int UG = 4;
+  const int UG = p.ug;
   const int ublk = wg / (UG * p.nob), r = wg % (UG * p.nob);
   const int gb = min(UG, p.total / p.nob - ublk * UG);  // units in this group (the last may hold fewer)
   const int unit = ublk * UG + r % gb;
@@ -414,6 +415,7 @@ void launch_pass(KParams p, uint64_t units, bool causal, hipStream_t st) {
   p.nob = (n_own + BO - 1) / BO;
   p.total = (int)(units * p.nob);
   p.per_xcd = (p.total + 7) / 8;
+  p.ug = std::max(4, (64 + p.nob - 1) / p.nob);  // enough units to fill an XCD's slots with one round
   const dim3 grid((unsigned)(p.per_xcd * 8)), block(256);
   if (p.bias) {
     if (causal) hipLaunchKernelGGL((fmha_bwd_kernel<T, HP, OWNER_K, true, DS, PV, true>), grid, block, 0, st, p);

@@ -20,6 +20,7 @@
 // 2^8 (so O is rescaled in few blocks), and O is divided by l once at the end.  Causal: key >
 // query masked (top-left aligned), key blocks past the diagonal are never visited, work-groups
 // are issued heaviest first.
+#include <algorithm>
 #include <utility>
 
 #include "common.h"
@@ -50,6 +51,7 @@ struct FmhaParams {
   int nqb;       // query blocks per unit
   int total;     // work-groups with work: units * nqb
   int per_xcd;   // ceil(total / 8)
+  int ug;        // units dealt together inside an XCD's range
   float scale2;  // head_scale * log2(e), > 0
 };
 
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   // Inside the range, units go four at a time, query blocks outermost and heaviest (latest) first: the four
   // units' work-groups of one causal weight are dealt together, so an XCD's slots run dry at about the same
   // time (unit by unit, the last unit's heaviest block would start when most slots are about to finish).
-  constexpr int UG = 4;  // measured: 1: 697, 2: 730, 4: 756, 8: 751, 16: 733, 32: 699 TFLOP/s on the causal [8,32,2048,128] case
+  const int UG = p.ug;
   const int ublk = wg / (UG * p.nqb), r = wg % (UG * p.nqb);
   const int gb = min(UG, p.total / p.nqb - ublk * UG);  // units in this group (the last may hold fewer)
   const int unit = ublk * UG + r % gb;
@@ -513,6 +515,9 @@ void launch_cfg(FmhaParams p, uint64_t units, uint32_t F, bool causal, int bias,
   p.nqb = (int)((F + NW * QT * 32 - 1) / (NW * QT * 32));
   p.total = (int)(units * p.nqb);
   p.per_xcd = (p.total + 7) / 8;
+  // Four units at a time (measured on causal [8,32,2048,128]: 1: 697, 2: 730, 4: 756, 8: 751, 16: 733, 32: 699
+  // TFLOP/s), more when a unit has so few query blocks that four units do not fill an XCD's 64 slots.
+  p.ug = std::max(4, (64 + p.nqb - 1) / p.nqb);
   const dim3 grid((unsigned)(p.per_xcd * 8)), block(NW * 64);
   // bias: 0 none, 1 element-wise from global memory, 2 staged through LDS
   if (causal) {
