@@ -90,7 +90,7 @@ def wl_fmha_bwd(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
     flops = 10.0 * B * N * S * S * H * (0.5 if causal else 1.0)
     return dict(name=f"fmha_bwd_{'causal_' if causal else ''}bf16_b{B}_h{N}_s{S}_d{H}",
                 fn=lambda: xmk.fmha_backward(q, k, v, out, d_o, lse, causal=causal), flops=flops,
-                bytes=10.0 * B * N * S * H * 2, bound="mfma", dtype="bf16", kernel="fmha_bwd_kernel (3 launches)",
+                bytes=10.0 * B * N * S * H * 2, bound="mfma", dtype="bf16", kernel="fmha_bwd_kernel (3 launches: dK, dV, dQ)",
                 note="flops counted as 5 matrix products (2.5x forward)")
 
 
