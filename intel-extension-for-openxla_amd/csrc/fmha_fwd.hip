@@ -481,31 +481,44 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
     if (it + 1 < nblk) block(it + 1, st_b, st_a, kst0, vst0 + TILE, kst0 + TILE, vst0, btile0);
   }
 
-  // ---- finish: O = O^T / l; LSE = m ln2 + ln l.
+  // ---- finish: O = O^T / l; LSE = m ln2 + ln l.  The accumulator layout gives a lane 8 bytes in each of 16
+  // places of its row, so the rounded rows go through LDS (free after the last block's barrier; one region of
+  // 32 rows per wave and query tile, 16-byte chunks XORed with the row so that both passes spread over the
+  // banks) and leave with 16-byte stores that cover whole rows.
+  constexpr int OCPR = HP / 8;  // 16-byte chunks per output row
+  static_assert(QT * NW * 32 * ROWB <= 4 * TILE, "the output tiles are staged in the K / V stages");
   static_for<QT>([&](auto TI) {
     constexpr int t = decltype(TI)::value;
     const int qrow = wq0 + 32 * t + l32;
     const float l_tot = l_run[t] + __shfl_xor(l_run[t], 32);
     const float inv = 1.0f / l_tot;
-    if (qrow < F) {
-      T* orow = reinterpret_cast<T*>(p.out) + ((int64_t)unit * F + qrow) * H;
-      static_for<HT>([&](auto HTI) {
-        constexpr int ht = decltype(HTI)::value;
-        const floatx16 o = ot[t][ht];
+    char* region = lds + (wave * QT + t) * (32 * ROWB);
+    static_for<HT>([&](auto HTI) {
+      constexpr int ht = decltype(HTI)::value;
+      const floatx16 o = ot[t][ht];
 #pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const int h = 32 * ht + 8 * qd + 4 * g;
-          if (h < H) {  // H % 8 == 0, so the four values are all in range
-            union { T e[4]; u32x2 w; } r;
-            r.e[0] = (T)(o[4 * qd + 0] * inv);
-            r.e[1] = (T)(o[4 * qd + 1] * inv);
-            r.e[2] = (T)(o[4 * qd + 2] * inv);
-            r.e[3] = (T)(o[4 * qd + 3] * inv);
-            *reinterpret_cast<u32x2*>(orow + h) = r.w;
-          }
-        }
-      });
-      if (p.lse && g == 0) p.lse[(int64_t)unit * F + qrow] = m_run[t] * 0.6931471805599453f + logf(l_tot);
+      for (int qd = 0; qd < 4; ++qd) {
+        union { T e[4]; u32x2 w; } r;
+        r.e[0] = (T)(o[4 * qd + 0] * inv);
+        r.e[1] = (T)(o[4 * qd + 1] * inv);
+        r.e[2] = (T)(o[4 * qd + 2] * inv);
+        r.e[3] = (T)(o[4 * qd + 3] * inv);
+        const int chunk = (4 * ht + qd) ^ (l32 & (OCPR - 1));
+        *reinterpret_cast<u32x2*>(region + l32 * ROWB + (chunk << 4) + g * 8) = r.w;
+      }
+    });
+    if (qrow < F && p.lse && g == 0) p.lse[(int64_t)unit * F + qrow] = m_run[t] * 0.6931471805599453f + logf(l_tot);
+    // this wave's own region: its LDS writes are complete for its own reads once lgkmcnt is zero
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(63));
+    constexpr int RPI = 64 / OCPR;  // rows per store instruction
+    const int c = lane % OCPR;
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const int row = it * RPI + lane / OCPR;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(region + row * ROWB + ((c ^ (row & (OCPR - 1))) << 4));
+      const int qr = wq0 + 32 * t + row;
+      if (qr < F && c * 8 < H)  // H % 8 == 0: a chunk lies inside the row or outside as a whole
+        *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(p.out) + ((int64_t)unit * F + qr) * H + c * 8) = v;
     }
   });
 }
