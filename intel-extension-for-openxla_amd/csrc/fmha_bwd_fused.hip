@@ -383,26 +383,37 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
     }
   }
 
-  // ---- store: acc^T[h][owner row] -> out[owner row][h]
-  if (orow < n_own) {
+  // ---- store: acc^T[h][owner row] -> out[owner row][h].  A lane holds 8 bytes in each of 16 places of its
+  // row; the rounded rows go through this wave's own LDS region (the stages are free after the last block's
+  // barrier), 16-byte chunks XORed with the row, and leave with 16-byte stores that cover whole rows.
+  {
+    constexpr int OCPR = HP / 8;  // 16-byte chunks per output row
+    static_assert(4 * 32 * ROWB <= 4 * TILE, "the output rows are staged in the tile stages");
+    char* region = lds + wave * (32 * ROWB);
     auto store = [&](void* out, const floatx16 (&acc)[HT], float mul) {
-      T* dst = reinterpret_cast<T*>(out) + ((int64_t)unit * n_own + orow) * H;
       static_for<HT>([&](auto HTI) {
         constexpr int ht = decltype(HTI)::value;
         const floatx16 o = acc[ht];
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
-          const int h = 32 * ht + 8 * qd + 4 * g;
-          if (h < H) {  // H % 8 == 0, so the four values are all in range
-            union { T e[4]; u32x2 w; } r;
-            r.e[0] = (T)(o[4 * qd + 0] * mul);
-            r.e[1] = (T)(o[4 * qd + 1] * mul);
-            r.e[2] = (T)(o[4 * qd + 2] * mul);
-            r.e[3] = (T)(o[4 * qd + 3] * mul);
-            *reinterpret_cast<u32x2*>(dst + h) = r.w;
-          }
+          union { T e[4]; u32x2 w; } r;
+          r.e[0] = (T)(o[4 * qd + 0] * mul);
+          r.e[1] = (T)(o[4 * qd + 1] * mul);
+          r.e[2] = (T)(o[4 * qd + 2] * mul);
+          r.e[3] = (T)(o[4 * qd + 3] * mul);
+          const int chunk = (4 * ht + qd) ^ (l32 & (OCPR - 1));
+          *reinterpret_cast<u32x2*>(region + l32 * ROWB + (chunk << 4) + g * 8) = r.w;
         }
       });
+      constexpr int RPI = 64 / OCPR;  // rows per store instruction
+      const int c = lane % OCPR;
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int row = it * RPI + lane / OCPR;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(region + row * ROWB + ((c ^ (row & (OCPR - 1))) << 4));
+        if (wo0 + row < n_own && c * 8 < H)  // H % 8 == 0: a chunk lies inside the row or outside as a whole
+          *reinterpret_cast<u32x4*>(reinterpret_cast<T*>(out) + ((int64_t)unit * n_own + wo0 + row) * H + c * 8) = v;
+      }
     };
     if constexpr (DS) store(p.out1, acc1, p.scale);
     if constexpr (PV) store(p.out2, acc2, 1.0f);
