@@ -405,9 +405,16 @@ extern "C" int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, 
                     xmk::aligned(b, 16) && xmk::aligned(out, 8) && 256 * k < (int64_t)kOob;
   if (fast) {
     const bool big = xmk::ceil_div(m, 256) * xmk::ceil_div(n, 256) >= 256;
+    // Between the two: about one 256 x 128 tile per CU (the 16-bit GEMM's third tile, for the same shapes).
+    static const char* tile_env = getenv("XMK_FP8_TILE");
+    const int64_t mid_tiles = xmk::ceil_div(m, 256) * xmk::ceil_div(n, 128);
+    const bool mid = tile_env ? atoi(tile_env) == 1 : (!big && mid_tiles >= 192 && mid_tiles <= 256);
     xmk::trace("fp8_gemm m=%lld n=%lld k=%lld -> %s", (long long)m, (long long)n, (long long)k,
-               big ? "mfma_256x256" : "mfma_128x128");
-    if (big) {
+               mid ? "mfma_256x128" : big ? "mfma_256x256" : "mfma_128x128");
+    if (mid) {
+      p.tiles_m = (int)xmk::ceil_div(m, 256); p.tiles_n = (int)xmk::ceil_div(n, 128);
+      hipLaunchKernelGGL((fp8_gemm_kernel<256, 128, 2, 2, 4>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
+    } else if (tile_env ? atoi(tile_env) == 2 : big) {
       p.tiles_m = (int)xmk::ceil_div(m, 256); p.tiles_n = (int)xmk::ceil_div(n, 256);
       hipLaunchKernelGGL((fp8_gemm_kernel<256, 256, 2, 4, 4>), dim3(p.tiles_m * p.tiles_n), dim3(512), 0, st, p);
     } else {

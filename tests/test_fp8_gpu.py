@@ -21,6 +21,8 @@ def _quant(oracle, shape, seed):
     (130, 72, 80, False), (256, 256, 256, False),
     # the gathering kernel: [k,n]-stored B, K that is not a multiple of 16, odd N, both tile sizes
     (300, 515, 1027, False), (37, 52, 45, True), (2100, 2060, 200, False), (2100, 2060, 72, True),
+    # about one 256 x 128 tile per CU: the third tile of the direct kernel, whole and with ragged edges
+    (2048, 4096, 128, True), (1800, 4000, 144, True),
 ])
 def test_fp8_gemm_shapes(xmk, oracle, m, n, k, rhs_t):
     a, sa = _quant(oracle, (m, k), 1)
