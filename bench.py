@@ -19,6 +19,7 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0}  # dense MFMA TFLOP/s, MI355X
 HBM_PEAK = 8000.0                                        # GB/s
+RAMP_SECONDS = 0.25                                      # untimed launches before the warmup steps (clock ramp)
 
 # HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (KiB per dispatch), FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0: the factors a
@@ -37,6 +38,14 @@ def _events(torch, fn, steps, warmup, graph=False):
     (the stream every xmk call below is launched on).  graph=True replays the launches from one
     captured HIP graph, so that kernels of a few microseconds are not timed at the rate the host
     can enqueue them from Python."""
+    # Bring the device to its sustained clocks first: from idle it takes about 50 ms of continuous
+    # work before the kernels run at their steady rate (the first 10 ms run at little more than half of
+    # it).  These launches are neither warmup steps nor timed steps.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < RAMP_SECONDS:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()

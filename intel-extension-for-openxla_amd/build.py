@@ -22,6 +22,11 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I", INCLUDE, "
          "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes"] + os.environ.get("XMK_CXXFLAGS", "").split()
 
 
+# Per-file flags.  fmha_fwd.hip: matrix instructions write VGPRs, so that the softmax reads the
+# scores where they were produced (the whole register budget is then one file of 256 per wave).
+EXTRA = {"fmha_fwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith((".hip", ".cc")))
 
@@ -39,7 +44,7 @@ def _compile(args):
     if (not force and os.path.exists(obj)
             and os.path.getmtime(obj) > max(os.path.getmtime(spath), _deps_mtime())):
         return src, obj, 0, ""
-    cmd = [HIPCC] + FLAGS + (["-x", "hip"] if src.endswith(".cc") else []) + \
+    cmd = [HIPCC] + FLAGS + EXTRA.get(src, []) + (["-x", "hip"] if src.endswith(".cc") else []) + \
           ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     out = "\n".join(l for l in (r.stdout + r.stderr).splitlines()

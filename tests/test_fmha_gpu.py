@@ -1,6 +1,11 @@
 """GPU parity: fused multi-head-attention forward through the C ABI (xmk_fmha_fwd) against the
-oracle's closed form.  Tolerance: max relative error <= 1e-2 (bf16/fp16), plus the reference
-test's own absolute bound (test/jax_ut.patch:997: atol 3e-2 bf16, 1e-2 fp16)."""
+oracle's closed form.  Tolerance 1e-2 (bf16/fp16) on (a) the error relative to the tensor's scale and
+(b) the error relative to sum_t p_t |v_t|, the scale of the terms each output is the sum of; plus the
+reference test's own absolute bound (test/jax_ut.patch:997: atol 3e-2 bf16, 1e-2 fp16).  The
+elementwise figure with eps = rms(ref) is held to 2e-2: P is rounded to the 16-bit type before P V
+(as the reference does, fmha_forward.h:378-384), and on the first causal rows, whose few O(1) terms
+are larger than the rms of the whole unit's output, that rounding alone reaches 1.3e-2 of rms(ref)
+in bf16 (measured on every kernel version; fp16 stays below 2e-3)."""
 import numpy as np
 import pytest
 import torch
@@ -35,8 +40,13 @@ def _run(xmk, oracle, name, B, N, F, T, H, *, causal=False, use_bias=False, lse=
         _, ref, ref_lse = oracle.fmha_fwd(q, k, v, dt, scale, bias=bias, causal=causal, want_lse=True,
                                           first_unit=u, num_units=1, f_stride=f_stride)
         ref = ref.reshape(B * N, F, H)[u, ::f_stride]
-        g, e = oracle.rel_err(got[u, ::f_stride], ref)
-        assert g <= 1e-2 and e <= 1e-2, (u, g, e)
+        _, ref_abs, _ = oracle.fmha_fwd(q, k, v & 0x7FFF, dt, scale, bias=bias, causal=causal,
+                                        first_unit=u, num_units=1, f_stride=f_stride)
+        ref_abs = ref_abs.reshape(B * N, F, H)[u, ::f_stride]
+        g, e = oracle.rel_err(got[u, ::f_stride], ref,
+                              label=f"fmha_fwd {name} [{B},{N},{F}x{T},{H}] causal={causal} bias={use_bias} unit {u}")
+        c = oracle.cond_err(got[u, ::f_stride], ref, ref_abs)
+        assert g <= 1e-2 and c <= 1e-2 and e <= 2e-2, (u, g, c, e)
         assert np.abs(got[u, ::f_stride] - ref).max() <= (3e-2 if name == "bf16" else 1e-2)
         if lse:
             gl = lse_t.cpu().numpy()[u, ::f_stride]
@@ -47,6 +57,15 @@ def _run(xmk, oracle, name, B, N, F, T, H, *, causal=False, use_bias=False, lse=
 def test_config2_causal_bf16(xmk, oracle):
     """benchmark configuration 2: bf16 [8,32,2048,128], causal, scale 1/sqrt(128); three units, every 8th row."""
     _run(xmk, oracle, "bf16", 8, 32, 2048, 2048, 128, causal=True, units=[0, 101, 255], f_stride=8)
+
+
+@pytest.mark.parametrize("H", [64, 128, 256])
+@pytest.mark.parametrize("causal,use_bias", [(False, True), (True, True), (True, False)])
+def test_many_key_tiles(xmk, oracle, H, causal, use_bias):
+    """32 key tiles, so that the unmasked steady-state steps of the pipeline run; the bias (in score units,
+    N(0,1)) makes the running reference max move in later tiles too, which exercises the deferred
+    rescale of O and of the row sum."""
+    _run(xmk, oracle, "bf16", 1, 2, 2048, 2048, H, causal=causal, use_bias=use_bias, lse=True, seed=31, f_stride=4)
 
 
 def test_config2_full_size_properties(xmk, oracle):
