@@ -180,6 +180,11 @@ int xmk_fmha_bwd(const void* query, const void* key, const void* value, const vo
 size_t xmk_fmha_decode_workspace_bytes(uint32_t num_batches, uint32_t num_heads,
                                        uint32_t head_size, uint32_t num_keys);
 
+/* Bytes of workspace that serve xmk_fmha_decode for EVERY num_keys in 1..cache_capacity (the split
+ * count is not monotonic in num_keys): what a caller that allocates once for a KV cache asks for. */
+size_t xmk_fmha_decode_cache_workspace_bytes(uint32_t num_batches, uint32_t num_heads,
+                                             uint32_t head_size, uint32_t cache_capacity);
+
 /* Attention for one query row per (batch, head) (num_queries == 1), with the
  * keys split over work-groups and merged by a second pass.  Same tensors as
  * xmk_fmha_fwd with F = 1; key/value may sit in a cache whose rows per head

@@ -66,6 +66,7 @@ def lib():
                               ("xmk_last_error", ctypes.c_char_p),
                               ("xmk_gemm_policy_name", ctypes.c_char_p),
                               ("xmk_fmha_decode_workspace_bytes", ctypes.c_size_t),
+                              ("xmk_fmha_decode_cache_workspace_bytes", ctypes.c_size_t),
                               ("xmk_fmha_bwd_workspace_bytes", ctypes.c_size_t),
                               ("xmk_gemm_workspace_bytes", ctypes.c_size_t),
                               ("xmk_int4_gemm_workspace_bytes", ctypes.c_size_t)):
@@ -187,6 +188,12 @@ def fmha_backward(query, key, value, out, grad_out, lse, *, bias=None, head_scal
 def fmha_decode_workspace_bytes(B, N, H, T):
     return lib().xmk_fmha_decode_workspace_bytes(ctypes.c_uint32(B), ctypes.c_uint32(N),
                                                  ctypes.c_uint32(H), ctypes.c_uint32(T))
+
+
+def fmha_decode_cache_workspace_bytes(B, N, H, capacity):
+    """Workspace that serves fmha_decode for every num_keys in 1..capacity."""
+    return lib().xmk_fmha_decode_cache_workspace_bytes(ctypes.c_uint32(B), ctypes.c_uint32(N),
+                                                       ctypes.c_uint32(H), ctypes.c_uint32(capacity))
 
 
 def fmha_decode(query, key, value, out, workspace, *, num_keys=None, kv_head_stride=None,

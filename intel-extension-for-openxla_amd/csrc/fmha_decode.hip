@@ -11,6 +11,8 @@
 // partial results and writes the output row.
 #include <cstdlib>
 
+#include <algorithm>
+
 #include "common.h"
 
 namespace {
@@ -252,25 +254,41 @@ extern "C" size_t xmk_fmha_decode_workspace_bytes(uint32_t num_batches, uint32_t
   return (size_t)units * splits * (head_size + 2) * sizeof(float);
 }
 
-extern "C" int xmk_fmha_decode(const void* query, const void* key, const void* value, void* out,
-                               int32_t dtype, uint32_t num_batches, uint32_t num_heads,
-                               uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
-                               float head_scale, void* workspace, size_t workspace_bytes,
-                               void* stream) {
+extern "C" size_t xmk_fmha_decode_cache_workspace_bytes(uint32_t num_batches, uint32_t num_heads,
+                                                        uint32_t head_size, uint32_t cache_capacity) {
+  // The split count is not monotonic in the number of keys (the chunk is rounded to 32 and clamped
+  // to 64..512 keys), so a cache is sized for the largest count any fill level 1..capacity plans.
+  const uint32_t units = num_batches * num_heads;
+  if (units == 0 || cache_capacity == 0) return 0;
+  int most = 0;
+  for (uint32_t t = 1; t <= cache_capacity; ++t) {
+    int splits, chunk;
+    plan(units, t, &splits, &chunk);
+    most = std::max(most, splits);
+  }
+  return (size_t)units * most * (head_size + 2) * sizeof(float);
+}
+
+namespace {
+
+int decode_checked(const void* query, const void* key, const void* value, void* out, int32_t dtype,
+                   uint32_t num_batches, uint32_t num_heads, uint32_t head_size, uint32_t num_keys,
+                   int64_t kv_head_stride, float head_scale, void* workspace, size_t workspace_bytes,
+                   const char* what, void* stream) {
   if (!query || !key || !value || !out || !workspace)
-    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: null pointer");
+    return xmk::fail(XMK_INVALID_ARGUMENT, "%s: null pointer", what);
   if (dtype != XMK_F16 && dtype != XMK_BF16) return xmk::fail(XMK_INTERNAL, "Invalid MHA datatype");
   if (num_batches == 0 || num_heads == 0 || head_size == 0 || num_keys == 0)
-    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: empty dimension");
+    return xmk::fail(XMK_INVALID_ARGUMENT, "%s: empty dimension", what);
   if (head_size > 256 || head_size % 8 != 0)
-    return xmk::fail(XMK_UNIMPLEMENTED, "fmha_decode: head_size must be a multiple of 8, at most 256");
+    return xmk::fail(XMK_UNIMPLEMENTED, "%s: head_size must be a multiple of 8, at most 256", what);
   if (kv_head_stride < (int64_t)num_keys * head_size || kv_head_stride % 8 != 0)
-    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: kv_head_stride too small or not a multiple of 8");
+    return xmk::fail(XMK_INVALID_ARGUMENT, "%s: kv_head_stride too small or not a multiple of 8", what);
   if (!xmk::aligned(query, 16) || !xmk::aligned(key, 16) || !xmk::aligned(value, 16))
-    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: tensors must be 16-byte aligned");
+    return xmk::fail(XMK_INVALID_ARGUMENT, "%s: tensors must be 16-byte aligned", what);
   const size_t need = xmk_fmha_decode_workspace_bytes(num_batches, num_heads, head_size, num_keys);
   if (workspace_bytes < need)
-    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_decode: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    return xmk::fail(XMK_INVALID_ARGUMENT, "%s: workspace of %zu bytes, %zu needed", what, workspace_bytes, need);
   DecodeParams p;
   p.q = query; p.k = key; p.v = value; p.out = out; p.ws = (float*)workspace;
   p.N = (int)num_heads; p.H = (int)head_size; p.T = (int)num_keys;
@@ -279,11 +297,22 @@ extern "C" int xmk_fmha_decode(const void* query, const void* key, const void* v
   const uint32_t units = num_batches * num_heads;
   plan(units, num_keys, &p.splits, &p.chunk);
   if (p.splits > MAXSPLITS)
-    return xmk::fail(XMK_UNIMPLEMENTED, "fmha_decode: %u keys need %d splits, more than %d", num_keys, p.splits,
+    return xmk::fail(XMK_UNIMPLEMENTED, "%s: %u keys need %d splits, more than %d", what, num_keys, p.splits,
                      MAXSPLITS);
-  xmk::trace("fmha_decode B=%u N=%u T=%u H=%u splits=%d chunk=%d", num_batches, num_heads, num_keys,
+  xmk::trace("%s B=%u N=%u T=%u H=%u splits=%d chunk=%d", what, num_batches, num_heads, num_keys,
              head_size, p.splits, p.chunk);
   if (dtype == XMK_BF16) launch<__bf16>(p, (int)units, (hipStream_t)stream);
   else launch<_Float16>(p, (int)units, (hipStream_t)stream);
-  return xmk::check_launch("fmha_decode");
+  return xmk::check_launch(what);
+}
+
+}  // namespace
+
+extern "C" int xmk_fmha_decode(const void* query, const void* key, const void* value, void* out,
+                               int32_t dtype, uint32_t num_batches, uint32_t num_heads,
+                               uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
+                               float head_scale, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  return decode_checked(query, key, value, out, dtype, num_batches, num_heads, head_size, num_keys,
+                        kv_head_stride, head_scale, workspace, workspace_bytes, "fmha_decode", stream);
 }

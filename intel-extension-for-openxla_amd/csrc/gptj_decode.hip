@@ -142,8 +142,9 @@ Workspace carve(const xmk_gptj_config& c, char* base) {
   w.q = (_Float16*)take(B * d * 2);
   w.attn = (_Float16*)take(B * d * 2);
   w.ff = (_Float16*)take(B * (size_t)c.d_ff * 2);
-  w.attn_ws_bytes = xmk_fmha_decode_workspace_bytes((uint32_t)c.batch, (uint32_t)c.n_head,
-                                                    (uint32_t)c.head_dim, (uint32_t)c.cache_capacity);
+  // sized for every fill level of the cache: a step attends to position + 1 <= cache_capacity keys
+  w.attn_ws_bytes = xmk_fmha_decode_cache_workspace_bytes((uint32_t)c.batch, (uint32_t)c.n_head,
+                                                          (uint32_t)c.head_dim, (uint32_t)c.cache_capacity);
   w.attn_ws = take(w.attn_ws_bytes);
   // fp32 partial sums of the K-split out_proj and fc_out GEMMs (when the plan splits them)
   w.ks_out = xmk::int4_plan_split(c.batch, c.d_model, c.d_model, c.group);

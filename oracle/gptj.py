@@ -25,9 +25,19 @@ def dequant_f32(qw, scales, zeros, group):
     return ((q - z).astype(np.float32) * s).astype(np.float32)
 
 
-def linear(x, lin, group):
+def predequantize(lin, group):
+    """A linear layer with its weight dequantised once (for tests that apply one layer many times)."""
     qw, s, z, b = lin
-    y = x @ dequant_f32(qw, s, z, group).astype(np.float64)
+    return {"dense": dequant_f32(qw, s, z, group), "bias": b}
+
+
+def linear(x, lin, group):
+    if isinstance(lin, dict):
+        y = (x.astype(np.float64) @ lin["dense"]).astype(np.float64)  # fp32 weights, float64 accumulate
+        b = lin["bias"]
+    else:
+        qw, s, z, b = lin
+        y = x @ dequant_f32(qw, s, z, group).astype(np.float64)
     if b is not None:
         y = y + to_f32(b, F16).astype(np.float64)
     return y

@@ -63,3 +63,19 @@ def test_null_arguments_are_rejected_before_any_device_work(lib):
                           ctypes.c_uint32(1), ctypes.c_uint32(64), ctypes.c_uint32(1), ctypes.c_uint32(1),
                           ctypes.c_float(1.0), ctypes.c_int32(0), None)
     assert rc == 3
+
+
+def test_decode_cache_workspace_covers_every_fill_level(lib):
+    """The split plan of the decode attention is not monotonic in the number of keys; the workspace a
+    cache is sized with must cover every fill level (e.g. 64 units: capacity 2050 plans 13 splits,
+    2048 keys plan 16)."""
+    lib.xmk_fmha_decode_workspace_bytes.restype = ctypes.c_size_t
+    lib.xmk_fmha_decode_cache_workspace_bytes.restype = ctypes.c_size_t
+    u32 = ctypes.c_uint32
+    for units, cap in ((64, 2050), (64, 1087), (64, 1025), (64, 2048), (8, 4097), (300, 777), (1, 70000)):
+        have = lib.xmk_fmha_decode_cache_workspace_bytes(u32(1), u32(units), u32(256), u32(cap))
+        step = max(1, cap // 3000)
+        worst = max(lib.xmk_fmha_decode_workspace_bytes(u32(1), u32(units), u32(256), u32(t))
+                    for t in list(range(1, cap + 1, step)) + [cap])
+        assert worst <= have, (units, cap, worst, have)
+        assert have <= 4 * lib.xmk_fmha_decode_workspace_bytes(u32(1), u32(units), u32(256), u32(cap)) + 64 * 258 * 4

@@ -60,15 +60,15 @@ def test_gptj_tiny_matches_transformers_fixture(xmk, oracle):
         assert g <= 3e-2 and e <= 3e-2, (pos, g, e)  # fp16 intermediates through 2 blocks vs fp32 torch
 
 
-@pytest.mark.parametrize("n_layer,position", [(2, 2047), (1, 0), (1, 300)])
-def test_gptj_full_width_vs_oracle(xmk, oracle, n_layer, position):
+@pytest.mark.parametrize("n_layer,position,cap", [(2, 2047, 2048), (1, 0, 2048), (1, 300, 2048), (1, 1023, 1087)])
+def test_gptj_full_width_vs_oracle(xmk, oracle, n_layer, position, cap):
     """benchmark configuration 5 at full width (d_model 4096, 16 heads x 256, rotary 64, MLP 16384, vocab
-    50400, batch 4, cache filled with N(0,1) to `position`), fewer blocks so the numpy oracle
-    finishes in seconds."""
+    50400, batch 4, cache of `cap` rows filled with N(0,1) to `position`), fewer blocks so the numpy
+    oracle finishes in seconds."""
     from oracle import gptj as og
     cfg = dict(n_layer=n_layer, n_head=16, head_dim=256, rotary_dim=64, d_model=4096, d_ff=16384,
                vocab=50400, group=128, ln_eps=1e-5)
-    B, cap = 4, 2048
+    B = 4  # (capacity 1087 with 1024 keys: a fill level that plans more key splits than the capacity itself)
     layers, lnf, lm_head = random_model(oracle, cfg, seed=3)
     dec, dl = _device_model(xmk, cfg, layers, lnf, lm_head, B, cap)
     hidden = oracle.from_f32(oracle.normal((B, cfg["d_model"]), 9), oracle.F16)
@@ -98,6 +98,46 @@ def test_gptj_full_width_vs_oracle(xmk, oracle, n_layer, position):
         assert np.abs(krow - kc[l][:, :, position]).max() <= 2e-2 * np.abs(kc[l][:, :, position]).max()
         vrow = dl[l]["v_cache"][:, :, position].float().cpu().numpy()
         assert np.abs(vrow - vc[l][:, :, position]).max() <= 2e-2 * np.abs(vc[l][:, :, position]).max()
+
+
+def test_gptj_28_layers_config5(xmk, oracle):
+    """benchmark configuration 5 at its full depth: 28 blocks, batch 4, 2047 cached keys.  To keep the
+    numpy oracle (and the host memory) within a test's budget the 28 blocks share one set of int4
+    weights and one K / V cache (each block appends its own row 2047 over the last one's, on the device
+    and in the oracle alike); every launch of the full-depth step runs at its real shape."""
+    from oracle import gptj as og
+    cfg = dict(n_layer=28, n_head=16, head_dim=256, rotary_dim=64, d_model=4096, d_ff=16384,
+               vocab=50400, group=128, ln_eps=1e-5)
+    B, cap, position = 4, 2048, 2047
+    one = dict(cfg, n_layer=1)
+    layers, lnf, lm_head = random_model(oracle, one, seed=5)
+    dec1, dl = _device_model(xmk, one, layers, lnf, lm_head, B, cap)
+    del dec1
+    c = xmk.GptjConfig(28, 16, 256, 64, 4096, 16384, 50400, 128, B, cap, 1e-5)
+
+    def lin(t):
+        qw, s, z, b = t
+        return (to_dev(qw, "u32"), to_dev(s, "f16"), to_dev(z, "f16"), None if b is None else to_dev(b, "f16"))
+    dec = xmk.GptjDecoder(c, [dl[0]] * 28, to_dev(lnf[0], "f16"), to_dev(lnf[1], "f16"), lin(lm_head))
+    hidden = oracle.from_f32(oracle.normal((B, 4096), 9, 0.5), oracle.F16)
+    kb = oracle.from_f32(oracle.normal((B, 16, cap, 256), 70), oracle.F16)
+    vb = oracle.from_f32(oracle.normal((B, 16, cap, 256), 71), oracle.F16)
+    dl[0]["k_cache"].copy_(to_dev(kb, "f16"))
+    dl[0]["v_cache"].copy_(to_dev(vb, "f16"))
+    logits = torch.empty((B, 50400), dtype=torch.float16, device="cuda")
+    dec.step(to_dev(hidden, "f16"), position, logits)
+    torch.cuda.synchronize()
+    got = logits.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    ol = as_oracle_layers(oracle, layers)[0]
+    ol = dict(ol, **{k: og.predequantize(ol[k], 128) for k in ("qkv", "out_proj", "fc_in", "fc_out")})
+    kc = oracle.to_f32(kb, oracle.F16).astype(np.float64)
+    vc = oracle.to_f32(vb, oracle.F16).astype(np.float64)
+    lnf64 = tuple(oracle.to_f32(x, oracle.F16).astype(np.float64) for x in lnf)
+    ref, _ = og.decode_step(cfg, [ol] * 28, lnf64, lm_head, oracle.to_f32(hidden, oracle.F16).astype(np.float64),
+                            [kc] * 28, [vc] * 28, position)
+    g, e = oracle.rel_err(got, ref, label="gptj decode step, 28 blocks, batch 4, 2047 cached keys")
+    assert g <= 1e-2 and e <= 1e-2
 
 
 def test_gptj_errors(xmk, oracle):
