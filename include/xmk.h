@@ -195,6 +195,21 @@ int xmk_fmha_decode(const void* query, const void* key, const void* value, void*
                     uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
                     float head_scale, void* workspace, size_t workspace_bytes, void* stream);
 
+/* xmk_fmha_decode for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): no workspace argument; the partial results of the
+ * key splits go to an array that is part of the library image on each GPU (4 MiB per GPU, held from
+ * the first call there until the process ends).  No counterpart in the reference.  Calls neither
+ * hipMalloc / hipFree nor any allocating routine; results equal xmk_fmha_decode's bit for bit.  Shapes
+ * whose xmk_fmha_decode_workspace_bytes() exceeds xmk_fmha_decode_static_max_bytes() are rejected with
+ * XMK_INVALID_ARGUMENT.  All calls on one GPU share that GPU's array: calls that overlap in time on
+ * one GPU (different streams, or threads) race; calls ordered on one stream are safe.  The device
+ * the stream belongs to must be the calling thread's current device. */
+size_t xmk_fmha_decode_static_max_bytes(void);
+int xmk_fmha_decode_static(const void* query, const void* key, const void* value, void* out,
+                           int32_t dtype, uint32_t num_batches, uint32_t num_heads,
+                           uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
+                           float head_scale, void* stream);
+
 /* Int4 weight-only GEMM (not in the reference snapshot; the contract is this
  * header's):
  *   qweight int32 [K/8, N]: nibble j (bits 4j..4j+3) of qweight[r, n] is the

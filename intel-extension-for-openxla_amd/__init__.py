@@ -67,6 +67,7 @@ def lib():
                               ("xmk_gemm_policy_name", ctypes.c_char_p),
                               ("xmk_fmha_decode_workspace_bytes", ctypes.c_size_t),
                               ("xmk_fmha_decode_cache_workspace_bytes", ctypes.c_size_t),
+                              ("xmk_fmha_decode_static_max_bytes", ctypes.c_size_t),
                               ("xmk_fmha_bwd_workspace_bytes", ctypes.c_size_t),
                               ("xmk_gemm_workspace_bytes", ctypes.c_size_t),
                               ("xmk_int4_gemm_workspace_bytes", ctypes.c_size_t)):
@@ -212,6 +213,26 @@ def fmha_decode(query, key, value, out, workspace, *, num_keys=None, kv_head_str
                                  ctypes.c_size_t(workspace.numel() * workspace.element_size()),
                                  _stream(stream)))
     return out
+
+
+def fmha_decode_static(query, key, value, out, *, num_keys=None, kv_head_stride=None, head_scale=None,
+                       stream=None):
+    """fmha_decode without a workspace argument: the key splits' partial results go to an array
+    inside the library image (xmk_fmha_decode_static: it allocates nothing)."""
+    B, N = query.shape[0], query.shape[1]
+    H = query.shape[-1]
+    T = key.shape[2] if num_keys is None else num_keys
+    stride = key.stride(1) if kv_head_stride is None else kv_head_stride
+    scale = (H ** -0.5) if head_scale is None else head_scale
+    _check(lib().xmk_fmha_decode_static(_ptr(query), _ptr(key), _ptr(value), _ptr(out),
+                                        ctypes.c_int32(dtype_code(query)), ctypes.c_uint32(B),
+                                        ctypes.c_uint32(N), ctypes.c_uint32(H), ctypes.c_uint32(T),
+                                        ctypes.c_int64(stride), ctypes.c_float(scale), _stream(stream)))
+    return out
+
+
+def fmha_decode_static_max_bytes():
+    return lib().xmk_fmha_decode_static_max_bytes()
 
 
 # ----------------------------------------------------------------------- int4

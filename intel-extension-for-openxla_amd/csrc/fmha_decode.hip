@@ -12,6 +12,7 @@
 #include <cstdlib>
 
 #include <algorithm>
+#include <atomic>
 
 #include "common.h"
 
@@ -315,4 +316,58 @@ extern "C" int xmk_fmha_decode(const void* query, const void* key, const void* v
                                void* stream) {
   return decode_checked(query, key, value, out, dtype, num_batches, num_heads, head_size, num_keys,
                         kv_head_stride, head_scale, workspace, workspace_bytes, "fmha_decode", stream);
+}
+
+// ---- The entry point that allocates nothing -------------------------------------------------
+// Same kernels as xmk_fmha_decode; the partial results of the key splits go to a device array that
+// is part of the library's code object instead of caller memory.  Every GPU holds its own copy of
+// the array, at its own address, from the first call on that GPU until the process ends.
+namespace {
+
+constexpr size_t kStaticScratchBytes = size_t{4} << 20;  // 4 MiB: config 5 (64 units, 16 splits, head size 256) needs 1.06 MB
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+std::atomic<float*> scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, once looked up
+
+// Device address of this GPU's copy of `scratch`.  The array's name is a host-side stand-in, not a
+// device address; the address comes from the runtime, once per device, with that device current.
+int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return xmk::fail(XMK_INTERNAL, "fmha_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return xmk::fail(XMK_INTERNAL, "fmha_decode_static: device index %d", dev);
+  float* p = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !addr)
+      return xmk::fail(XMK_INTERNAL, "fmha_decode_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    p = static_cast<float*>(addr);
+    scratch_ptr[dev].store(p, std::memory_order_release);  // concurrent first calls store the same address
+  }
+  *out = p;
+  return XMK_OK;
+}
+
+}  // namespace
+
+extern "C" size_t xmk_fmha_decode_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int xmk_fmha_decode_static(const void* query, const void* key, const void* value, void* out,
+                                      int32_t dtype, uint32_t num_batches, uint32_t num_heads,
+                                      uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
+                                      float head_scale, void* stream) {
+  const size_t need = xmk_fmha_decode_workspace_bytes(num_batches, num_heads, head_size, num_keys);
+  if (need > kStaticScratchBytes)
+    return xmk::fail(XMK_INVALID_ARGUMENT,
+                     "fmha_decode_static: this shape needs %zu bytes of scratch, the built-in array holds %zu; "
+                     "use xmk_fmha_decode with a workspace", need, kStaticScratchBytes);
+  float* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != XMK_OK) return rc;
+  // Every partial result the merge kernel reads is written by the split kernel of the same call, so
+  // nothing needs clearing between calls.
+  return decode_checked(query, key, value, out, dtype, num_batches, num_heads, head_size, num_keys,
+                        kv_head_stride, head_scale, ws, kStaticScratchBytes, "fmha_decode_static", stream);
 }
