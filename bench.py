@@ -189,24 +189,8 @@ def wl_copy(torch, xmk, nbytes=1 << 30):
                 bound="hbm", dtype="u8", kernel="torch copy kernel")
 
 
-def wl_mfma_probe(torch, xmk, tile, iters=2048, fp8=False):
-    """Nothing but MFMA instructions on every SIMD of the device: the rate the matrix cores sustain
-    under the board's power limit, to read the kernels' fractions of the published peak against."""
-    sink = torch.empty((1 << 18,), dtype=torch.float32, device="cuda")
-    dt = xmk.F8E4M3FN if fp8 else xmk.BF16
-    flops = xmk.probe_mfma_rate(sink, dtype=dt, tile=tile, iters=1)
-    shape = f"{tile}x{tile}x{(16 if tile == 32 else 32) * (4 if fp8 else 1)}"
-    return dict(name=f"mfma_only_loop_{'fp8' if fp8 else 'bf16'}_{shape}",
-                fn=lambda: xmk.probe_mfma_rate(sink, dtype=dt, tile=tile, iters=iters),
-                flops=flops * iters, bytes=0.0, bound="mfma", dtype="fp8" if fp8 else "bf16", kernel="mfma_rate_kernel")
-
-
 WORKLOADS = {
     "copy": lambda t, x: wl_copy(t, x),
-    "mfma_probe_32": lambda t, x: wl_mfma_probe(t, x, 32),
-    "mfma_probe_16": lambda t, x: wl_mfma_probe(t, x, 16),
-    "mfma_probe_fp8_32": lambda t, x: wl_mfma_probe(t, x, 32, fp8=True),
-    "mfma_probe_fp8_16": lambda t, x: wl_mfma_probe(t, x, 16, fp8=True),
     "fmha_causal": lambda t, x: wl_fmha(t, x, True),
     "fmha": lambda t, x: wl_fmha(t, x, False),
     "fmha_bwd_causal": lambda t, x: wl_fmha_bwd(t, x, True),
@@ -220,8 +204,7 @@ WORKLOADS = {
     "fp8_8192": lambda t, x: wl_fp8(t, x, 8192, 8192, 8192),
     "gptj_decode": lambda t, x: wl_gptj_decode(t, x),
 }
-ALSO = ["fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "gptj_decode",
-        "mfma_probe_32", "mfma_probe_16", "mfma_probe_fp8_32", "mfma_probe_fp8_16"]
+ALSO = ["fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "gptj_decode"]
 
 
 def measure(torch, xmk, key, steps, warmup):

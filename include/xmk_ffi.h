@@ -43,6 +43,16 @@ XLA_FFI_Error* xmk_ffi_cublas_lt_matmul(XLA_FFI_CallFrame* call_frame);
 XLA_FFI_Error* xmk_ffi_fmha_softmax(XLA_FFI_CallFrame* call_frame);
 XLA_FFI_Error* xmk_ffi_fmha_scale_bias_softmax(XLA_FFI_CallFrame* call_frame);
 
+/* "__cudnn$fmhaSoftmaxBackward" / "__cudnn$fmhaScaleBiasSoftmaxBackward": replace
+ * RunXetlaGpuFMHABackward (xetla_gpu_fused_mha_runner.cc:419-445; kinds dispatched at :404-416).
+ * operands, in the runner's order: (Q, K, activation f32 [B,N,F] as written by the forward call, V,
+ * d_output [, bias [B,N,F,T]], fwd_output) -> results (dQ, dK, dV [, scratch ...]).  Attributes as
+ * for the forward targets.  Needs a host API table with XLA_FFI_DeviceMemory_Allocate / _Free (the
+ * reference takes its dp_sum / accumulation buffers from the thunk's scratch, :392-399).  The
+ * operand order the compiler emits is fixed in a patch that is not part of the reference tree. */
+XLA_FFI_Error* xmk_ffi_fmha_softmax_backward(XLA_FFI_CallFrame* call_frame);
+XLA_FFI_Error* xmk_ffi_fmha_scale_bias_softmax_backward(XLA_FFI_CallFrame* call_frame);
+
 /* "__xmk$int4_gemm" (no counterpart in the reference): operands (act f16 [M,K], qweight s32|u32
  * [K/8,N], scales f16 [K/g,N], zeros f16 [K/g,N] [, bias f16 [N]]) -> results (out f16 [M,N]);
  * the group size is K / scales.dims[0]. */

@@ -279,16 +279,6 @@ def fp8_gemm(a, b, a_scale, b_scale, out, *, rhs_transpose=False, stream=None):
     return out
 
 
-# ---------------------------------------------------------------------- probe
-def probe_mfma_rate(sink, *, dtype=BF16, tile=32, iters=1024, stream=None):
-    """xmk_probe_mfma_rate: a device-wide loop of MFMA instructions only; returns the flops of the call."""
-    L = lib()
-    L.xmk_probe_mfma_flops.restype = ctypes.c_double
-    _check(L.xmk_probe_mfma_rate(ctypes.c_int32(dtype), ctypes.c_int32(tile), ctypes.c_int32(iters), _ptr(sink),
-                                 ctypes.c_uint64(sink.numel() * sink.element_size()), _stream(stream)))
-    return float(L.xmk_probe_mfma_flops(ctypes.c_int32(dtype), ctypes.c_int32(tile), ctypes.c_int32(iters)))
-
-
 # ------------------------------------------------------------ GPT-J decode step
 class Int4Linear(ctypes.Structure):
     """xmk_int4_linear."""

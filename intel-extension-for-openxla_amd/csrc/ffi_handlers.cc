@@ -288,11 +288,67 @@ XLA_FFI_Error* fmha_common(XLA_FFI_CallFrame* f, bool with_bias) {
                                  (uint32_t)N, (uint32_t)H, (uint32_t)F, (uint32_t)T, scale, causal, stream));
 }
 
+// Backward kinds (CudnnfMHAKind::kBackwardSoftmax / kBackwardScaleBiasSoftmax, dispatched at
+// xetla_gpu_fused_mha_runner.cc:404-416).  Operands in the runner's order (:419-433):
+// bmm1_grad_gemm1_rhs = Q, bmm1_grad_gemm2_rhs = K, bmm2_grad_gemm1_lhs = the forward activation
+// (log-sum-exp, f32 [B,N,F]), bmm2_grad_gemm2_rhs = V, d_output [, bias], fwd_output.
+// Results: d_bmm1_lhs = dQ, d_bmm1_rhs = dK, d_bmm2_rhs = dV [, scratch ...]; d_s and d_bias are not
+// produced (the reference passes d_bias on but its kernel never writes it, :383-385).
+XLA_FFI_Error* fmha_bwd_common(XLA_FFI_CallFrame* f, bool with_bias) {
+  if (metadata_query(f) || f->stage != XLA_FFI_ExecutionStage_EXECUTE) return nullptr;
+  Frame fr{f};
+  const XLA_FFI_Buffer* q = fr.arg(0);
+  const XLA_FFI_Buffer* k = fr.arg(1);
+  const XLA_FFI_Buffer* act = fr.arg(2);
+  const XLA_FFI_Buffer* v = fr.arg(3);
+  const XLA_FFI_Buffer* d_out = fr.arg(4);
+  const XLA_FFI_Buffer* bias = with_bias ? fr.arg(5) : nullptr;
+  const XLA_FFI_Buffer* fwd_out = fr.arg(with_bias ? 6 : 5);
+  const XLA_FFI_Buffer* dq = fr.ret(0);
+  const XLA_FFI_Buffer* dk = fr.ret(1);
+  const XLA_FFI_Buffer* dv = fr.ret(2);
+  if (fr.code != XMK_OK) return finish(fr, XMK_OK);
+  if (fr.has("dropout_rate") && fr.f64("dropout_rate") != 0.0)
+    fr.fail(XMK_UNIMPLEMENTED, "Unimplemented dropout");  // :244-250
+  const int64_t rank = q->rank;
+  if ((rank != 3 && rank != 4) || k->rank != rank || v->rank != rank || d_out->rank != rank || fwd_out->rank != rank)
+    fr.fail(XMK_INVALID_ARGUMENT, "fmha backward: operands must all have rank 3 or 4");
+  if (fr.code != XMK_OK) return finish(fr, XMK_OK);
+  const int64_t B = rank == 4 ? q->dims[0] : 1;
+  const int64_t N = q->dims[rank - 3], F = q->dims[rank - 2], H = q->dims[rank - 1];
+  const int64_t T = k->dims[rank - 2];
+  if (k->dims[rank - 1] != H || v->dims[rank - 1] != H || v->dims[rank - 2] != T || k->dims[rank - 3] != N ||
+      v->dims[rank - 3] != N || elements(d_out) != B * N * F * H || elements(fwd_out) != B * N * F * H ||
+      elements(act) != B * N * F || elements(dq) != B * N * F * H || elements(dk) != B * N * T * H ||
+      elements(dv) != B * N * T * H || (bias && elements(bias) != B * N * F * T))
+    fr.fail(XMK_INVALID_ARGUMENT, "fmha backward: operand shapes do not agree");
+  for (const XLA_FFI_Buffer* b : {k, v, d_out, fwd_out, dq, dk, dv})
+    if (b->dtype != q->dtype) fr.fail(XMK_INVALID_ARGUMENT, "fmha backward: operand types do not agree");
+  if (bias && bias->dtype != q->dtype) fr.fail(XMK_INVALID_ARGUMENT, "fmha backward: operand types do not agree");
+  if (act->dtype != XLA_FFI_DataType_F32) fr.fail(XMK_INVALID_ARGUMENT, "fmha backward: activation must be f32");
+  float scale = fr.has("fmha_scale") ? (float)fr.f64("fmha_scale") : 1.0f;
+  if ((scale - 1.0f) > 1e-6f) scale = 1.0f / std::sqrt((float)H);  // as in the forward handler
+  const int causal = fr.has("is_causal_mask") ? (int)fr.i64("is_causal_mask") : 0;
+  void* stream = fr.stream();
+  if (fr.code != XMK_OK) return finish(fr, XMK_OK);
+  // dp_sum / grad_query_accum of the reference (:392-399) are one workspace here, from the
+  // executor's scratch allocator.
+  const size_t need = xmk_fmha_bwd_workspace_bytes((uint32_t)B, (uint32_t)N, (uint32_t)H, (uint32_t)F, (uint32_t)T);
+  return finish(fr, with_scratch(f, need, [&](void* ws) {
+    if (!ws) return xmk::fail(XMK_INTERNAL, "fmha backward: the host's API table has no scratch allocator");
+    return xmk_fmha_bwd(q->data, k->data, v->data, bias ? bias->data : nullptr, fwd_out->data, d_out->data,
+                        static_cast<const float*>(act->data), dq->data, dk->data, dv->data, (int32_t)q->dtype,
+                        (uint32_t)B, (uint32_t)N, (uint32_t)H, (uint32_t)F, (uint32_t)T, scale, causal, ws, need, stream);
+  }));
+}
+
 const xmk_ffi_target kTargets[] = {
     {"__cublas$gemm", xmk_ffi_cublas_gemm},
     {"__cublas$lt$matmul", xmk_ffi_cublas_lt_matmul},
     {"__cudnn$fmhaSoftmax", xmk_ffi_fmha_softmax},
     {"__cudnn$fmhaScaleBiasSoftmax", xmk_ffi_fmha_scale_bias_softmax},
+    {"__cudnn$fmhaSoftmaxBackward", xmk_ffi_fmha_softmax_backward},
+    {"__cudnn$fmhaScaleBiasSoftmaxBackward", xmk_ffi_fmha_scale_bias_softmax_backward},
     {"__xmk$int4_gemm", xmk_ffi_int4_gemm},
     {"__cublas$lt$matmul$f8", xmk_ffi_cublas_lt_matmul_f8},
 };
@@ -303,6 +359,10 @@ extern "C" XLA_FFI_Error* xmk_ffi_cublas_gemm(XLA_FFI_CallFrame* f) { return gem
 extern "C" XLA_FFI_Error* xmk_ffi_cublas_lt_matmul(XLA_FFI_CallFrame* f) { return gemm_common(f, true); }
 extern "C" XLA_FFI_Error* xmk_ffi_fmha_softmax(XLA_FFI_CallFrame* f) { return fmha_common(f, false); }
 extern "C" XLA_FFI_Error* xmk_ffi_fmha_scale_bias_softmax(XLA_FFI_CallFrame* f) { return fmha_common(f, true); }
+extern "C" XLA_FFI_Error* xmk_ffi_fmha_softmax_backward(XLA_FFI_CallFrame* f) { return fmha_bwd_common(f, false); }
+extern "C" XLA_FFI_Error* xmk_ffi_fmha_scale_bias_softmax_backward(XLA_FFI_CallFrame* f) {
+  return fmha_bwd_common(f, true);
+}
 
 extern "C" XLA_FFI_Error* xmk_ffi_int4_gemm(XLA_FFI_CallFrame* f) {
   if (metadata_query(f) || f->stage != XLA_FFI_ExecutionStage_EXECUTE) return nullptr;

@@ -125,6 +125,19 @@ int gemm(const xmk_matrix& lhs, const xmk_matrix& rhs, const xmk_matrix& out, in
   return xmk_gemm(&d, stream);
 }
 
+// Whether the fused kernels take the call (they need only the rowsum(dO o O) part of the workspace).
+// A bias is assumed when `bias` is unknown (the workspace query): its size only tightens the test.
+bool fused_path(uint64_t units, uint32_t H, uint32_t F, uint32_t T, bool maybe_bias) {
+  static const bool composed = getenv("XMK_FMHA_BWD_COMPOSED") != nullptr;
+  if (composed) return false;
+  fmha_bwd_fused::Args a{};
+  a.H = (int)H; a.F = (int)F; a.T = (int)T;
+  a.bias = maybe_bias ? &a : nullptr;  // any non-null value: only its presence is looked at
+  return fmha_bwd_fused::eligible(a, units);
+}
+
+size_t dsum_bytes(uint64_t units, uint64_t F) { return ((size_t)units * F * sizeof(float) + 255) & ~(size_t)255; }
+
 template <typename T>
 int run(const void* q, const void* k, const void* v, const void* bias, const void* o, const void* d_o,
         const float* lse, void* dq, void* dk, void* dv, int dtype, int64_t units, int64_t H, int64_t F, int64_t Tk,
@@ -148,9 +161,8 @@ int run(const void* q, const void* k, const void* v, const void* bias, const voi
   // The gradients come from the fused kernels, which keep the scores on chip;
   // XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
   {
-    static const bool composed = getenv("XMK_FMHA_BWD_COMPOSED") != nullptr;
     const fmha_bwd_fused::Args a{q, k, v, d_o, bias, lse, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
-    if (!composed && fmha_bwd_fused::eligible(a, (uint64_t)units)) {
+    if (fused_path((uint64_t)units, (uint32_t)H, (uint32_t)F, (uint32_t)Tk, bias != nullptr)) {
       fmha_bwd_fused::launch(a, (uint64_t)units, dtype == XMK_BF16, st);
       return xmk::check_launch("fmha_bwd");
     }
@@ -198,7 +210,10 @@ int check_dims(uint32_t B, uint32_t N, uint32_t H, uint32_t F, uint32_t T) {
 extern "C" size_t xmk_fmha_bwd_workspace_bytes(uint32_t num_batches, uint32_t num_heads, uint32_t head_size,
                                                uint32_t num_queries, uint32_t num_keys) {
   if (check_dims(num_batches, num_heads, head_size, num_queries, num_keys) != XMK_OK) return 0;
-  return make_plan((uint64_t)num_batches * num_heads, num_queries, num_keys).total;
+  const uint64_t units = (uint64_t)num_batches * num_heads;
+  // The fused kernels keep the scores on chip; only the GEMM composition needs the score-sized buffers.
+  if (fused_path(units, head_size, num_queries, num_keys, true)) return dsum_bytes(units, num_queries);
+  return make_plan(units, num_queries, num_keys).total;
 }
 
 extern "C" int xmk_fmha_bwd(const void* query, const void* key, const void* value, const void* bias,
@@ -217,8 +232,10 @@ extern "C" int xmk_fmha_bwd(const void* query, const void* key, const void* valu
     return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_bwd: head_scale must be positive and finite");
   const uint64_t units = (uint64_t)num_batches * num_heads;
   const Plan pl = make_plan(units, num_queries, num_keys);
-  if (workspace_bytes < pl.total)
-    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_bwd: workspace of %zu bytes, %zu needed", workspace_bytes, pl.total);
+  const size_t need = fused_path(units, head_size, num_queries, num_keys, bias != nullptr) ? dsum_bytes(units, num_queries)
+                                                                                          : pl.total;
+  if (workspace_bytes < need)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_bwd: workspace of %zu bytes, %zu needed", workspace_bytes, need);
   if (pl.chunk > 65535) return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_bwd: shape too large");
   if (!xmk::aligned(workspace, 256) || !xmk::aligned(query, 16) || !xmk::aligned(key, 16) ||
       !xmk::aligned(value, 16) || !xmk::aligned(out, 16) || !xmk::aligned(grad_out, 16) ||

@@ -1,12 +1,12 @@
 // bf16 / fp16 GEMM with fp32 accumulation and a fused epilogue:
 //     out = act(alpha * op(lhs) op(rhs) + beta * c + bias)
 //
-// MFMA kernel (gemm_mfma_kernel): one work-group owns a BM x BN tile of the output
-// and walks K in steps of 64.  Operand tiles go from global memory straight into LDS
-// (buffer_load ... lds, 16 bytes per lane, no staging registers and no ds_write): a wave's
-// load fills 1 KiB of contiguous LDS, and the per-lane *global* address is chosen so that
-// the data lands swizzled.  Two LDS stages; the loads of K step t+1 are issued between the
-// MFMAs of step t and are waited for only at the single barrier per step.
+// MFMA kernel (gemm_mfma_kernel): one work-group owns a BM x BN tile of the output and walks K in
+// steps of BK (32 for the 256x256 tile, 64 for the smaller ones).  Operand tiles go from global memory
+// straight into LDS (buffer_load ... lds, 16 bytes per lane, no staging registers and no ds_write): a
+// wave's load fills 1 KiB of contiguous LDS, and the per-lane *global* address is chosen so that the
+// data lands swizzled.  A ring of three or four LDS stages; the loads of later K steps are issued
+// between the MFMAs of step t and are waited for with a counted s_waitcnt at the one barrier per step.
 //   "KC" operand (reduction index contiguous in memory: A[M,K] row-major, B stored [N,K]):
 //       LDS [row][64 k], the 16-byte chunks of a row XOR-swizzled by the row number, read
 //       with one ds_read_b128 per fragment.
@@ -271,6 +271,11 @@ extern "C" int xmk_gemm_ws(const xmk_gemm_desc* d, void* workspace, size_t works
     case XMK_EPI_BIAS_GELU: wants_bias = true; act = ACT_GELU; break;
     default: return run_gemm(d, nullptr, nullptr, stream);  // reports the error
   }
+  // (the sliced copy would hide a reduction size that differs between the operands, or a leading
+  // dimension shorter than the full row)
+  const int64_t k_rhs = d->rhs.transpose ? d->rhs.num_cols : d->rhs.num_rows;
+  if (k_rhs != k || d->lhs.leading_dim_stride < d->lhs.num_cols || d->rhs.leading_dim_stride < d->rhs.num_cols)
+    return run_gemm(d, nullptr, nullptr, stream);  // reports the error
   if ((wants_bias && !d->bias) || (d->beta != 0.0f && !d->c) || !d->out.data ||
       d->out.num_rows != m || d->out.num_cols != n || d->out.leading_dim_stride < n ||
       (d->dtype_out != d->dtype_in && d->dtype_out != XMK_F32))
@@ -360,6 +365,10 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
   if (m > INT32_MAX / 2 || n > INT32_MAX / 2 || k > INT32_MAX / 2 || d->batch_size > 65535)
     return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: dimension too large");
   if (!d->bias && wants_bias) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: bias missing");
+  // The tile loaders form byte offsets of up to 256 rows of an operand in 32 bits.
+  constexpr int64_t kMaxLd = int64_t{1} << 22;
+  if (lhs.leading_dim_stride >= kMaxLd || rhs.leading_dim_stride >= kMaxLd || out.leading_dim_stride >= kMaxLd)
+    return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: leading_dim_stride of 2^22 elements or more");
 
   hipStream_t st = (hipStream_t)stream;
   const bool qkv = out1 != nullptr;

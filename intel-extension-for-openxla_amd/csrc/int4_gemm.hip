@@ -171,7 +171,8 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   const __amdgpu_buffer_rsrc_t r_w = make_rsrc(qw, (uint32_t)((size_t)(K / 8) * N * 4));
   const __amdgpu_buffer_rsrc_t r_s = make_rsrc(scales, (uint32_t)((size_t)ngroups * N * 2));
   const __amdgpu_buffer_rsrc_t r_z = make_rsrc(zeros, (uint32_t)((size_t)ngroups * N * 2));
-  const __amdgpu_buffer_rsrc_t r_a = make_rsrc(act + (size_t)m_base * K, (uint32_t)((size_t)(M - m_base) * K * 2));
+  // (the 32 rows of this launch only: the byte count must fit the descriptor's 32 bits for any M)
+  const __amdgpu_buffer_rsrc_t r_a = make_rsrc(act + (size_t)m_base * K, (uint32_t)((size_t)min(M - m_base, 32) * K * 2));
   const uint32_t voff_w = col_ok ? (uint32_t)((kg * N + n0) * 4) : kOob;
   const uint32_t voff_sz = col_ok ? (uint32_t)(n0 * 2) : kOob;
   uint32_t voff_a[MT];
@@ -431,6 +432,10 @@ int prepare(const xmk::Int4Call& c, int64_t m, int64_t group, Config* cfg) {
     return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   if (k > (1 << 24) || n > (1 << 24) || m > (1 << 24))
     return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: dimension too large");
+  // The kernel addresses the packed weights, the scales and the zero points with 32-bit byte offsets.
+  if ((uint64_t)(k / 8) * (uint64_t)n * 4 >= (1ull << 31))
+    return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: packed weights of 2 GiB or more (k=%lld n=%lld)", (long long)k,
+                     (long long)n);
   if (!xmk::aligned(c.act, 16) || !xmk::aligned(c.qweight, 16) || !xmk::aligned(c.scales, 8) ||
       !xmk::aligned(c.zeros, 8) || !xmk::aligned(c.out, 2))
     return xmk::fail(XMK_INVALID_ARGUMENT, "int4_gemm: act, qweight must be 16-byte and scales, zeros 8-byte aligned");

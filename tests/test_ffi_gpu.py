@@ -20,7 +20,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def ffi():
     lib = C.CDLL(os.path.join(ROOT, "intel-extension-for-openxla_amd", "libxmk.so"))
     for name in ("xmk_ffi_cublas_gemm", "xmk_ffi_cublas_lt_matmul", "xmk_ffi_fmha_softmax",
-                 "xmk_ffi_fmha_scale_bias_softmax", "xmk_ffi_int4_gemm", "xmk_ffi_cublas_lt_matmul_f8"):
+                 "xmk_ffi_fmha_scale_bias_softmax", "xmk_ffi_int4_gemm", "xmk_ffi_cublas_lt_matmul_f8",
+                 "xmk_ffi_fmha_softmax_backward", "xmk_ffi_fmha_scale_bias_softmax_backward"):
         getattr(lib, name).restype = C.c_void_p
         getattr(lib, name).argtypes = [C.POINTER(F.CallFrame)]
     return lib
@@ -118,6 +119,54 @@ def test_fmha_handlers(ffi, oracle, with_bias, rank):
     g, e = oracle.rel_err(out.float().cpu().numpy().reshape(ref.shape), ref)
     assert g <= 1e-2 and e <= 1e-2, (g, e)
     assert np.abs(act.cpu().numpy().reshape(lse.shape) - lse).max() <= 2e-2
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_fmha_backward_handlers(ffi, oracle, with_bias):
+    """Forward handler (training call: writes the activation) then the backward handler on its results,
+    gradients against the oracle's float64 closed form; the workspace comes from the fake host's
+    allocator and goes back to it."""
+    B, N, Fq, T, H = 2, 3, 136, 200, 64
+    dt = oracle.BF16
+    q = oracle.from_f32(oracle.normal((B, N, Fq, H), 30), dt)
+    k = oracle.from_f32(oracle.normal((B, N, T, H), 31), dt)
+    v = oracle.from_f32(oracle.normal((B, N, T, H), 32), dt)
+    g = oracle.from_f32(oracle.normal((B, N, Fq, H), 33), dt)
+    bias = oracle.from_f32(oracle.normal((B, N, Fq, T), 34), dt) if with_bias else None
+    scale = H ** -0.5
+    rq, rk, rv = oracle.fmha_bwd(q, k, v, g, dt, scale, bias=bias, causal=True)
+    tq, tk, tv, tg = (to_dev(x, "bf16") for x in (q, k, v, g))
+    tb = to_dev(bias, "bf16") if with_bias else None
+    out = torch.empty_like(tq)
+    act = torch.empty((B, N, Fq), dtype=torch.float32, device="cuda")
+    scratch = torch.empty((16,), dtype=torch.uint8, device="cuda")
+    attrs = {"fmha_scale": (F.F64, scale), "dropout_rate": (F.F64, 0.0), "is_causal_mask": (F.S32, 1)}
+    host = _host()
+    f = host.frame([_buf(tq, F.BF16), _buf(tk, F.BF16), _buf(tv, F.BF16)] + ([_buf(tb, F.BF16)] if with_bias else []),
+                   [_buf(out, F.BF16), _buf(scratch, 6), _buf(act, F.F32)], attrs)
+    _ok(host, (ffi.xmk_ffi_fmha_scale_bias_softmax if with_bias else ffi.xmk_ffi_fmha_softmax)(C.byref(f)))
+
+    def allocator(size, alignment):
+        t = torch.empty((size + alignment,), dtype=torch.uint8, device="cuda")
+        return (t.data_ptr() + alignment - 1) // alignment * alignment, t
+    dq, dk, dv = torch.empty_like(tq), torch.empty_like(tk), torch.empty_like(tv)
+    host = F.FakeHost(stream=torch.cuda.current_stream().cuda_stream, allocator=allocator)
+    f = host.frame([_buf(tq, F.BF16), _buf(tk, F.BF16), _buf(act, F.F32), _buf(tv, F.BF16), _buf(tg, F.BF16)]
+                   + ([_buf(tb, F.BF16)] if with_bias else []) + [_buf(out, F.BF16)],
+                   [_buf(dq, F.BF16), _buf(dk, F.BF16), _buf(dv, F.BF16), _buf(scratch, 6)], attrs)
+    handler = ffi.xmk_ffi_fmha_scale_bias_softmax_backward if with_bias else ffi.xmk_ffi_fmha_softmax_backward
+    _ok(host, handler(C.byref(f)))
+    assert len(host.allocations) == 1 and host.freed == [host.allocations[0][0]]
+    assert host.allocations[0][0] <= 2 * B * N * Fq * 4 + 512  # the fused kernels need rowsum(dO o O) only
+    for name, got, ref in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+        ge, ee = oracle.rel_err(got.float().cpu().numpy(), ref.astype(np.float32))
+        assert ge <= 1e-2 and ee <= 8e-2, (name, ge, ee)
+    # a host without an allocator cannot run the backward call
+    host = _host()
+    f = host.frame([_buf(tq, F.BF16), _buf(tk, F.BF16), _buf(act, F.F32), _buf(tv, F.BF16), _buf(tg, F.BF16)]
+                   + ([_buf(tb, F.BF16)] if with_bias else []) + [_buf(out, F.BF16)],
+                   [_buf(dq, F.BF16), _buf(dk, F.BF16), _buf(dv, F.BF16), _buf(scratch, 6)], attrs)
+    assert handler(C.byref(f)) is not None and "scratch allocator" in host.errors[-1][1]
 
 
 def test_fmha_scale_above_one_is_recomputed(ffi, oracle):

@@ -15,6 +15,8 @@ TARGETS = {
     "__cublas$lt$matmul": "xmk_ffi_cublas_lt_matmul",
     "__cudnn$fmhaSoftmax": "xmk_ffi_fmha_softmax",
     "__cudnn$fmhaScaleBiasSoftmax": "xmk_ffi_fmha_scale_bias_softmax",
+    "__cudnn$fmhaSoftmaxBackward": "xmk_ffi_fmha_softmax_backward",
+    "__cudnn$fmhaScaleBiasSoftmaxBackward": "xmk_ffi_fmha_scale_bias_softmax_backward",
     "__xmk$int4_gemm": "xmk_ffi_int4_gemm",
     "__cublas$lt$matmul$f8": "xmk_ffi_cublas_lt_matmul_f8",
 }
