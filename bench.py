@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Roofline benchmark of the custom-call kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also] [--no-cpu] [--ramp S]
 
 One JSON line on stdout.  A "step" is one launch of the workload's kernel on synthetic inputs that
 are already resident in HBM.  The headline workload is benchmark configuration 2 (fused causal MHA forward,
@@ -222,20 +222,119 @@ def measure(torch, xmk, key, steps, warmup):
     return w, ms, wall_ms, roof
 
 
-def cpu_baseline_fmha(units=256, B=8, N=32, S=2048, H=128):
-    """The oracle (a CPU port of the path) on `units` of the workload's B*N (batch, head) units."""
-    import numpy as np
+def _cpu_time(fn, warm, timed):
+    for _ in range(warm):
+        fn()
+    t0 = time.perf_counter()
+    for _ in range(timed):
+        fn()
+    return (time.perf_counter() - t0) / timed
+
+
+def cpu_baseline(torch):
+    """The reference's CPU path for each benchmark configuration, as torch-CPU formulas (jax / jaxlib,
+    whose XLA-CPU backend the reference would use, is not installed): a bounded sample of each workload,
+    fp32 arithmetic on the rounded inputs, all host threads torch uses.  A reported baseline, not a
+    target.  The headline entry is configuration 2; the others are listed under "also"."""
+    try:
+        import jax  # noqa: F401
+        backend = "jax is importable but the harness times torch-CPU formulas"
+    except Exception:
+        backend = "torch-CPU formulas (jax not installed)"
+    threads = torch.get_num_threads()
+    g = torch.Generator().manual_seed(0)
+    out = {}
+    # C2: softmax(mask(Q K^T scale)) V on `units` of the 256 (batch, head) units
+    units, S, H = 64, 2048, 128
+    q, k, v = (torch.randn((units, S, H), generator=g).bfloat16().float() for _ in range(3))
+    mask = torch.ones((S, S), dtype=torch.bool).tril()
+
+    def attn():
+        s = torch.baddbmm(torch.zeros(()), q, k.transpose(1, 2), beta=0.0, alpha=H ** -0.5)
+        s.masked_fill_(~mask, float("-inf"))
+        return torch.softmax(s, -1) @ v
+    dt = _cpu_time(attn, 1, 3)
+    head = {"value": round(2.0 * units * S * S * H / dt / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "seconds": round(dt, 3), "backend": backend, "os_cpu_count": os.cpu_count(), "torch_num_threads": threads,
+            "sample": f"{units} of 256 (batch, head) units of the causal S=2048 D=128 workload, fp32 softmax(mask(QK^T/sqrt(D)))V "
+                      f"with causal FLOPs counted as 2*S^2*D per unit"}
+    # C1: a @ b + bias, whole problem
+    m, n, kk = 512, 4096, 4096
+    a, b, bias = torch.randn((m, kk), generator=g), torch.randn((kk, n), generator=g), torch.randn((n,), generator=g)
+    dt = _cpu_time(lambda: torch.addmm(bias, a, b), 3, 5)
+    out["gemm_bf16_512x4096x4096_bias"] = {"value": round(2.0 * m * n * kk / dt / 1e12, 4), "unit": "TFLOP/s",
+                                           "sample": "whole problem, fp32 addmm, 3 warm + 5 timed", "seconds": round(dt, 4)}
+    # C1b / C4: 8192^3 is sampled as 1024 rows of A against the whole B (the fp8 one upcasts e4m3 first)
+    m, n, kk = 1024, 8192, 8192
+    a, b = torch.randn((m, kk), generator=g), torch.randn((kk, n), generator=g)
+    dt = _cpu_time(lambda: a @ b, 1, 1)
+    out["gemm_bf16_8192x8192x8192"] = {"value": round(2.0 * m * n * kk / dt / 1e12, 4), "unit": "TFLOP/s",
+                                       "sample": "1024 of 8192 rows of A against the whole B, fp32 matmul, 1 warm + 1 timed",
+                                       "seconds": round(dt, 3)}
+    a8, b8 = a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn)
+    dt = _cpu_time(lambda: ((a8.float() @ b8.float()) * 0.5).bfloat16(), 1, 1)
+    out["gemm_fp8_e4m3_8192x8192x8192"] = {"value": round(2.0 * m * n * kk / dt / 1e12, 4), "unit": "TFLOP/s",
+                                           "sample": "1024 of 8192 rows of A: upcast e4m3 -> fp32, matmul, scale, round to bf16",
+                                           "seconds": round(dt, 3)}
+    # C3: unpack -> dequant -> dot, whole problem
+    kk, n, grp = 4096, 16384, 128
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (kk // 8, n), dtype=torch.int32, generator=g)
+    sc = (torch.rand((kk // grp, n), generator=g) * 0.019 + 0.001).half().float()
+    zp = (torch.rand((kk // grp, n), generator=g) * 15).half().float()
+    shifts = (torch.arange(8, dtype=torch.int32) * 4).view(1, 8, 1)
+
+    def int4(act):
+        qv = ((qw.unsqueeze(1) >> shifts) & 15).reshape(kk, n).float()
+        w = (qv - zp.repeat_interleave(grp, 0)) * sc.repeat_interleave(grp, 0)
+        return act @ w
+    for mm in (1, 8, 32):
+        act = torch.randn((mm, kk), generator=g).half().float()
+        dt = _cpu_time(lambda: int4(act), 1, 2)
+        nbytes = kk * n / 2 + 2 * (kk // grp) * n * 2 + 2 * mm * kk + 2 * mm * n
+        out[f"int4_gemm_m{mm}_k4096_n16384_g128"] = {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s",
+                                                    "sample": "whole problem: unpack, dequantise, fp32 matmul; 1 warm + 2 timed",
+                                                    "seconds": round(dt, 3)}
+    # C5: one decoder block of the 28 (its four int4 linears at batch 4 + attention over 2048 cached keys)
+    d, dff, heads, hd, B, T = 4096, 16384, 16, 256, 4, 2048
+    lin = {}
+    for name, (ki, ni) in {"qkv": (d, 3 * d), "out": (d, d), "fc_in": (d, dff), "fc_out": (dff, d)}.items():
+        lin[name] = (torch.randint(-2 ** 31, 2 ** 31 - 1, (ki // 8, ni), dtype=torch.int32, generator=g),
+                     (torch.rand((ki // grp, ni), generator=g) * 0.019 + 0.001).half().float(),
+                     (torch.rand((ki // grp, ni), generator=g) * 15).half().float())
+    kc, vc = torch.randn((B, heads, T, hd), generator=g), torch.randn((B, heads, T, hd), generator=g)
+    x = torch.randn((B, d), generator=g)
+
+    def dq(name):
+        qw_, sc_, zp_ = lin[name]
+        qv = ((qw_.unsqueeze(1) >> shifts) & 15).reshape(qw_.shape[0] * 8, qw_.shape[1]).float()
+        return (qv - zp_.repeat_interleave(grp, 0)) * sc_.repeat_interleave(grp, 0)
+
+    def block():
+        h = torch.nn.functional.layer_norm(x, (d,))
+        qkv = h @ dq("qkv")
+        qh = qkv[:, :d].view(B, heads, 1, hd)
+        p = torch.softmax((qh @ kc.transpose(-1, -2)) * hd ** -0.5, -1)
+        att = (p @ vc).reshape(B, d)
+        return x + att @ dq("out") + torch.nn.functional.gelu(h @ dq("fc_in"), approximate="tanh") @ dq("fc_out")
+    dt = _cpu_time(block, 0, 1)
+    out["gptj6b_decode_step_int4_l28_b4_kv2047"] = {"value": round(dt * 28 * 1e3, 1), "unit": "ms per step (28 x the one block timed)",
+                                                    "sample": "1 of 28 decoder blocks (lm_head left out): dequantise + fp32 matmul per "
+                                                              "linear, attention over 2048 cached keys; 1 timed",
+                                                    "seconds": round(dt, 3)}
+    head["also"] = out
+    return head
+
+
+def cpu_baseline_oracle(units=32, S=2048, H=128):
+    """The C oracle (double accumulation, OpenMP) on a sample of the headline workload, for comparison."""
     import oracle
-    rng_shape = (1, units, S, H)
-    q, k, v = (oracle.from_f32(oracle.normal(rng_shape, 5 + i), oracle.BF16) for i in range(3))
+    q, k, v = (oracle.from_f32(oracle.normal((1, units, S, H), 5 + i), oracle.BF16) for i in range(3))
     t0 = time.perf_counter()
     oracle.fmha_fwd(q, k, v, oracle.BF16, H ** -0.5, causal=True)
     dt = time.perf_counter() - t0
-    flops = 2.0 * units * S * S * H
-    return {"value": round(flops / dt / 1e12, 6), "unit": "TFLOP/s", "cores": oracle.num_threads(),
+    return {"value": round(2.0 * units * S * S * H / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(),
             "kind": "port", "seconds": round(dt, 2),
-            "sample": f"{units} of {B * N} (batch, head) units of the same causal bf16 "
-                      f"S={S} D={H} workload, oracle/xmk_oracle.c xo_fmha_fwd (OpenMP, double accumulation)"}
+            "sample": f"{units} of 256 units, oracle/xmk_oracle.c xo_fmha_fwd (OpenMP, double accumulation)"}
 
 
 def main():
@@ -246,12 +345,15 @@ def main():
     ap.add_argument("--workload", default="fmha_causal", choices=sorted(WORKLOADS))
     ap.add_argument("--no-also", action="store_true", help="time only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--ramp", type=float, default=RAMP_SECONDS,
+                    help="seconds of untimed launches before the warmup steps (0 for profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1",
               file=sys.stderr)
         sys.exit(2)
 
+    globals()["RAMP_SECONDS"] = args.ramp
     import torch
     xmk = importlib.import_module("intel-extension-for-openxla_amd")
     xmk.lib()  # fails loudly if libxmk.so is missing: there is no fallback path
@@ -276,7 +378,8 @@ def main():
             also[w2["name"]] = roof2
         line["also"] = also
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline_fmha()
+        line["cpu_baseline"] = cpu_baseline(torch)
+        line["cpu_baseline"]["also"]["oracle_fmha_fwd_causal"] = cpu_baseline_oracle()
     try:
         props = torch.cuda.get_device_properties(0)
         line["device"] = {"name": props.name, "cus": props.multi_processor_count,

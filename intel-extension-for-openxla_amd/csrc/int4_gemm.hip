@@ -8,7 +8,9 @@
 // core; nothing is staged through LDS.  Zero points and scales are applied once
 // per quantisation group on the fp32 accumulator:
 //     out[m,n] = sum_g s[g,n] * ( sum_{k in g} a[m,k] q[k,n]  -  z[g,n] * sum_{k in g} a[m,k] )
-// where the second sum comes from one extra MFMA against a B operand of ones.  The kernel
+// where the second sum comes from one extra MFMA against a B operand of ones, and the offsets the
+// unpack trick leaves on q are taken out by starting each group's accumulators at
+// -sum_k a[m,k] offset_k (one more extra MFMA, against a constant fragment).  The kernel
 // is bound by HBM only if the per-weight VALU work stays near one operation, so the
 // nibbles are expanded with the fp16 "magic number" trick (5 operations per 8 weights).
 #include <cstdlib>
@@ -41,8 +43,9 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t m
 // One packed word -> 8 fp16 values q + offset, in k-slot order (0,4,1,5,2,6,3,7):
 // 0x6400 | q is 1024 + q (slots 0,1,4,5) and 0x5400 | (q << 4) is 64 + q (slots 2,3,6,7).
 // The offsets are not subtracted here (that would cost as many VALU operations again);
-// they are removed per quantisation group through sum_k a_k * offset_k, which one extra
-// MFMA against a constant fragment provides.  5 VALU operations per 8 weights.
+// they are removed per quantisation group through -sum_k a_k * offset_k, which one extra
+// MFMA against a constant fragment provides as the accumulators' start value.  5 VALU operations
+// per 8 weights.
 __device__ __forceinline__ half8 unpack_word(uint32_t w, uint32_t m1024, uint32_t m64) {
   const uint32_t w8 = w >> 8;
   Frag f;
@@ -189,11 +192,11 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
 #pragma unroll
     for (int c = 0; c < W; ++c) acc[mt][c] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  Frag ones, offs;  // B operands that yield sum_k a_k and sum_k a_k * offset_k
+  Frag ones, noffs;  // B operands that yield sum_k a_k and -sum_k a_k * offset_k
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     ones.u[i] = 0x3c003c00u;
-    offs.u[i] = (i & 1) ? 0x54005400u : 0x64006400u;
+    noffs.u[i] = (i & 1) ? 0xd400d400u : 0xe400e400u;  // -64, -1024
   }
   uint32_t m1024 = 0x64006400u, m64 = 0x54005400u;
   asm volatile("" : "+v"(m1024), "+v"(m64));  // keep the magic constants in VGPRs
@@ -221,33 +224,36 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
       d.w[s] = load_words<W>(r_w, voff_w, (uint32_t)((g * 4 * SPG + s * 4) * N * 4));
   };
   auto compute = [&](const GroupData& cur) {
-    floatx4 d[MT][W], asum[MT], aoff[MT];
+    floatx4 d[MT][W], asum[MT], noff[MT];
+    half8 a[SPG][MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       asum[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-      aoff[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < W; ++c) d[mt][c] = floatx4{0.f, 0.f, 0.f, 0.f};
+      noff[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
+    // -sum_k a_k offset_k of the whole group first: it is the start value of every column's
+    // accumulator chain, so that the chains end at sum_k a_k q_k with the unpack offsets gone.
+#pragma unroll
+    for (int s = 0; s < SPG; ++s)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        a[s][mt] = permute_act(cur.a[s][mt]);
+        noff[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s][mt], noffs.h, noff[mt], 0, 0, 0);
+      }
 #pragma unroll
     for (int s = 0; s < SPG; ++s) {
-      half8 a[MT];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) a[mt] = permute_act(cur.a[s][mt]);
 #pragma unroll
       for (int c = 0; c < W; ++c) {
         const half8 b = unpack_word(cur.w[s].w[c], m1024, m64);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          d[mt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], b, d[mt][c], 0, 0, 0);
+          d[mt][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s][mt], b, s == 0 ? noff[mt] : d[mt][c], 0, 0, 0);
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        asum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], ones.h, asum[mt], 0, 0, 0);
-        aoff[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], offs.h, aoff[mt], 0, 0, 0);
-      }
+      for (int mt = 0; mt < MT; ++mt)
+        asum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s][mt], ones.h, asum[mt], 0, 0, 0);
     }
-    // acc += s * (sum a (q + off) - sum a off - z sum a), only for rows that can exist
+    // acc += s * (sum a q - z sum a), only for rows that can exist
 #pragma unroll
     for (int c = 0; c < W; ++c) {
       const float sc = half_at(cur.sc, c), z = half_at(cur.zp, c);
@@ -256,7 +262,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
 #pragma unroll
         for (int i = 0; i < RI; ++i) {
           const int e = i * ESTEP;
-          acc[mt][c][e] = fmaf(sc, d[mt][c][e] - fmaf(z, asum[mt][e], aoff[mt][e]), acc[mt][c][e]);
+          acc[mt][c][e] = fmaf(sc, fmaf(-z, asum[mt][e], d[mt][c][e]), acc[mt][c][e]);
         }
     }
   };
