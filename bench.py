@@ -115,16 +115,17 @@ def wl_gemm(torch, xmk, m, n, k, bias=False, rhs_t=False):
                 bound="mfma", dtype="bf16", kernel="gemm_mfma_kernel")
 
 
-def wl_fp8(torch, xmk, m, n, k):
+def wl_fp8(torch, xmk, m, n, k, rhs_t=True):
     a = torch.randn((m, k), device="cuda")
-    b = torch.randn((n, k), device="cuda")
+    b = torch.randn((n, k) if rhs_t else (k, n), device="cuda")
     sa, sb = a.abs().max() / 448.0, b.abs().max() / 448.0
     qa, qb = (a / sa).to(torch.float8_e4m3fn), (b / sb).to(torch.float8_e4m3fn)
     sa, sb = sa.reshape(1).float(), sb.reshape(1).float()
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
-    return dict(name=f"gemm_fp8_e4m3_{m}x{n}x{k}_rhsT", fn=lambda: xmk.fp8_gemm(qa, qb, sa, sb, out, rhs_transpose=True),
+    return dict(name=f"gemm_fp8_e4m3_{m}x{n}x{k}{'_rhsT' if rhs_t else '_rhs_kn'}",
+                fn=lambda: xmk.fp8_gemm(qa, qb, sa, sb, out, rhs_transpose=rhs_t),
                 flops=2.0 * m * n * k, bytes=1.0 * (m * k + k * n) + 2.0 * m * n, bound="mfma", dtype="fp8",
-                kernel="fp8_gemm_kernel")
+                kernel="fp8_gemm_kernel" if rhs_t else "fp8_gemm_gather_kernel")
 
 
 def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
@@ -181,6 +182,16 @@ def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
                 graph=True, graph_steps=3)
 
 
+def wl_lib_gemm(torch, xmk, m=8192, n=8192, k=8192):
+    """torch.matmul (hipBLASLt / rocBLAS behind it) on the 8192^3 shape: what the vendor library reaches on
+    the same device in the same run, to read the GEMM kernel's fraction of the published peak against."""
+    a = (torch.randn((m, k), device="cuda") * k ** -0.5).bfloat16()
+    b = (torch.randn((k, n), device="cuda") * k ** -0.5).bfloat16()
+    out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    return dict(name=f"library_torch_matmul_bf16_{m}x{n}x{k}", fn=lambda: torch.matmul(a, b, out=out), flops=2.0 * m * n * k,
+                bytes=2.0 * (m * k + k * n + m * n), bound="mfma", dtype="bf16", kernel="vendor library GEMM (not this library)")
+
+
 def wl_copy(torch, xmk, nbytes=1 << 30):
     """A plain device copy of known size: the calibration point for the HBM byte counters."""
     src = torch.empty((nbytes,), dtype=torch.uint8, device="cuda").random_(0, 255)
@@ -198,13 +209,15 @@ WORKLOADS = {
     "gemm_8192": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192),
     "gemm_8192_rhsT": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192, rhs_t=True),
     "gemm_c1": lambda t, x: wl_gemm(t, x, 512, 4096, 4096, bias=True),
+    "lib_gemm_8192": lambda t, x: wl_lib_gemm(t, x),
     "int4_m1": lambda t, x: wl_int4(t, x, 1),
     "int4_m8": lambda t, x: wl_int4(t, x, 8),
     "int4_m32": lambda t, x: wl_int4(t, x, 32),
     "fp8_8192": lambda t, x: wl_fp8(t, x, 8192, 8192, 8192),
+    "fp8_8192_kn": lambda t, x: wl_fp8(t, x, 8192, 8192, 8192, rhs_t=False),
     "gptj_decode": lambda t, x: wl_gptj_decode(t, x),
 }
-ALSO = ["fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "gptj_decode"]
+ALSO = ["fmha", "fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "lib_gemm_8192", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "fp8_8192_kn", "gptj_decode"]
 
 
 def measure(torch, xmk, key, steps, warmup):
