@@ -26,7 +26,7 @@ RAMP_SECONDS = 0.25                                      # untimed launches befo
 # 1 GiB device copy (--workload copy) gives on this machine.  The runs are summarised in
 # profiles/hbm_traffic_pmc.txt; a workload without a measurement reports null.
 TRAFFIC_BYTES = {
-    "fmha_causal": (196700 * 2.0 + 131100) * 1024,
+    "fmha_causal": (224900 * 2.0 + 131100) * 1024,
     "gemm_8192": (791700 * 2.0 + 131100) * 1024,
     "int4_m1": (17480 * 2.0 + 32) * 1024,
     "fp8_8192": (393600 * 2.0 + 131100) * 1024,
