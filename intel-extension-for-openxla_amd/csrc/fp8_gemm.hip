@@ -8,7 +8,9 @@
 // swizzle and wait/barrier scheme as the 16-bit GEMM: a 64-byte fp8 row is byte for byte
 // the 32-element 16-bit row that kernel's loader handles.  The per-tensor scales are read
 // from device memory in the epilogue.
-// B stored [K,N] (rhs_transpose == 0) runs a plain tiled kernel.
+// B stored [K,N] (rhs_transpose == 0) takes the same kernel: its 64 k x BN tile goes into LDS as it
+// lies in memory (n contiguous, the 16-bit GEMM's loader for that layout) and the fragments are read
+// with ds_read_b64_tr_b8, which hands a lane 8 consecutive k of one column.
 #include <utility>
 
 #include "gemm_gather8.h"
@@ -58,12 +60,45 @@ struct Fp8Frag {
   }
 };
 
+// The same fragments from a tile stored [64 k][BN columns] (row = BN bytes, 16-byte chunks XOR-swizzled
+// by the loader with swz<true, BN / 2, 64>(k)).  ds_read_b64_tr_b8 works on blocks of 16 lanes: lane p
+// of a block addresses row kb + p / 2, bytes cb + 8 (p % 2) .. +7 and receives column cb + p, rows
+// kb .. kb + 7.  Blocks 0 and 1 of the wave cover columns 0..15 and 16..31 of the slab for k half 0,
+// blocks 2 and 3 the same columns for k half 1; four reads, 8 rows apart, give a lane its 32 k.  The
+// swizzle depends on k & 7 = p / 2 only, so one address per slab serves the four reads.
+template <int BN, int T>
+struct Fp8FragKN {
+  int base[T];
+  __device__ __forceinline__ void init(int col0, int lane) {
+    const int p = lane & 15;
+    const int k = (lane >> 5) * 32 + (p >> 1);
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const int col = col0 + t * 32 + ((lane >> 4) & 1) * 16 + 8 * (p & 1);
+      base[t] = k * BN + (((col >> 4) ^ gemm_impl::swz<true, BN / 2, 64>(k)) << 4) + (col & 15);
+    }
+  }
+  // t counts 32-column slabs from col0; only slabs this wave owns are read.
+  __device__ __forceinline__ intx8 read(const char* __restrict__ tile, int t) const {
+    typedef int int2v __attribute__((ext_vector_type(2)));
+    typedef int2v __attribute__((address_space(3))) * lds_ptr;
+    intx8 v;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int2v r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr)(tile + base[t] + q * 8 * BN));
+      v[2 * q] = r[0];
+      v[2 * q + 1] = r[1];
+    }
+    return v;
+  }
+};
+
 __device__ __forceinline__ floatx16 mfma_fp8(intx8 a, intx8 b, floatx16 c) {
   // cbsz = blgp = 0: both operands e4m3; block scales 127 = 2^0 (E8M0).
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 127, 0, 127);
 }
 
-template <int BM, int BN, int WGM, int WGN, int NSTAGE>
+template <int BM, int BN, int WGM, int WGN, int NSTAGE, bool BKN = false>
 __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
   constexpr int NWAVES = WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -71,7 +106,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
   constexpr int A_BYTES = BM * BKB, B_BYTES = BN * BKB, STAGE = A_BYTES + B_BYTES;
   // The loader works in 2-byte units: BK = 32 units = 64 bytes.
   typedef gemm_impl::Loader<false, BM, 32, NWAVES> LoaderA;
-  typedef gemm_impl::Loader<false, BN, 32, NWAVES> LoaderB;
+  // B [n,k]: BN rows of 64 bytes; B [k,n]: 64 rows of BN bytes (BN / 2 two-byte units).
+  typedef std::conditional_t<BKN, gemm_impl::Loader<true, BN / 2, 64, NWAVES>, gemm_impl::Loader<false, BN, 32, NWAVES>>
+      LoaderB;
   constexpr int LOADS = LoaderA::NL + LoaderB::NL;  // per wave per K step
   static_assert(NSTAGE >= 3, "the barrier leaves the running step's loads in flight");
   __shared__ __attribute__((aligned(1024))) char lds[NSTAGE * STAGE];
@@ -100,9 +137,14 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
   LoaderA la;
   LoaderB lb;
   la.init(p.K / 2, p.M - m0, wave, lane);
-  lb.init(p.K / 2, p.N - n0, wave, lane);
+  if constexpr (BKN) lb.init(p.N / 2, (p.N - n0) / 2, wave, lane);
+  else lb.init(p.K / 2, p.N - n0, wave, lane);
   const uint8_t* a_tile = p.a + (int64_t)m0 * p.K;
-  const uint8_t* b_tile = p.b + (int64_t)n0 * p.K;
+  const uint8_t* b_tile = BKN ? p.b + n0 : p.b + (int64_t)n0 * p.K;
+  const int64_t b_step = BKN ? (int64_t)BKB * p.N : BKB;  // bytes from one K step's B tile to the next
+  // k of a K step that exist, in the unit the loader compares with: two-byte units along a
+  // k-contiguous row, rows of the [k,n] tile.
+  auto kleft_b = [&](int st) { return BKN ? p.K - st * BKB : (p.K - st * BKB) / 2; };
   const int KT = (p.K + BKB - 1) / BKB;
 
   // Prologue: K steps 0 .. NSTAGE-2.  Loads past the end of K write zeros, so every step issues
@@ -110,14 +152,15 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
 #pragma unroll
   for (int st = 0; st < NSTAGE - 1; ++st) {
     la.issue(a_tile, (p.K - st * BKB) / 2, lds + st * STAGE, wave);
-    lb.issue(b_tile, (p.K - st * BKB) / 2, lds + st * STAGE + A_BYTES, wave);
+    lb.issue(b_tile, kleft_b(st), lds + st * STAGE + A_BYTES, wave);
     a_tile += BKB;
-    b_tile += BKB;
+    b_tile += b_step;
   }
   __builtin_amdgcn_s_waitcnt(gemm_impl::vmcnt_imm((NSTAGE - 2) * LOADS));  // step 0 has landed
   __builtin_amdgcn_s_barrier();
 
-  Fp8Frag fa_addr, fb_addr;
+  Fp8Frag fa_addr;
+  std::conditional_t<BKN, Fp8FragKN<BN, TN>, Fp8Frag> fb_addr;
   fa_addr.init(wm * WTM, lane);
   fb_addr.init(wn * WTN, lane);
   // Fragment registers: the B fragments of a step are double-buffered (those of step kt + 1 are
@@ -142,7 +185,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
 #pragma unroll
     for (int i = 0; i < LoaderA::NL; ++i) la.issue_one(i, ra, kleft, wr, wave);
 #pragma unroll
-    for (int i = 0; i < LoaderB::NL; ++i) lb.issue_one(i, rb, kleft, wr + A_BYTES, wave);
+    for (int i = 0; i < LoaderB::NL; ++i) lb.issue_one(i, rb, kleft_b(kt + NSTAGE - 1), wr + A_BYTES, wave);
     static_for<TM>([&](auto I) {
       constexpr int i = decltype(I)::value;
       if constexpr (i + 1 < TM) fa[(i + 1) & 1] = fa_addr.read(cur, i + 1);
@@ -155,13 +198,13 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
     // are spread evenly.
     static_for<NMFMA>([&](auto R) {
       constexpr int r = decltype(R)::value;
-      if constexpr (r % TN == 0) __builtin_amdgcn_sched_group_barrier(0x100, (r / TN < TN) ? 4 : 2, 0);
+      if constexpr (r % TN == 0) __builtin_amdgcn_sched_group_barrier(0x100, (r / TN < TN) ? (BKN ? 6 : 4) : 2, 0);
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       if constexpr ((r + 1) * LOADS / NMFMA > r * LOADS / NMFMA) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
     });
     __builtin_amdgcn_sched_barrier(0);
     a_tile += BKB;
-    b_tile += BKB;
+    b_tile += b_step;
   };
 
 #pragma unroll
@@ -401,25 +444,31 @@ extern "C" int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, 
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.a_scale = a_scale; p.b_scale = b_scale;
   p.out = (__bf16*)out; p.M = (int)m; p.N = (int)n; p.K = (int)k;
   hipStream_t st = (hipStream_t)stream;
-  const bool fast = rhs_transpose != 0 && k % 16 == 0 && n % 4 == 0 && xmk::aligned(a, 16) &&
-                    xmk::aligned(b, 16) && xmk::aligned(out, 8) && 256 * k < (int64_t)kOob;
-  if (fast) {
+  // The direct-to-LDS kernel: A rows and the stored rows of B start on 16-byte boundaries and hold whole
+  // 16-byte chunks; one K step's tile of either operand lies within the 2 GiB a buffer descriptor spans.
+  const bool fast_nk = rhs_transpose != 0 && k % 16 == 0 && n % 4 == 0 && 256 * k < (int64_t)kOob;
+  const bool fast_kn = rhs_transpose == 0 && k % 16 == 0 && n % 16 == 0 && 256 * k < (int64_t)kOob &&
+                       64 * n < (int64_t)kOob;
+  if ((fast_nk || fast_kn) && xmk::aligned(a, 16) && xmk::aligned(b, 16) && xmk::aligned(out, 8)) {
     const bool big = xmk::ceil_div(m, 256) * xmk::ceil_div(n, 256) >= 256;
     // Between the two: about one 256 x 128 tile per CU (the 16-bit GEMM's third tile, for the same shapes).
     static const char* tile_env = getenv("XMK_FP8_TILE");
     const int64_t mid_tiles = xmk::ceil_div(m, 256) * xmk::ceil_div(n, 128);
     const bool mid = tile_env ? atoi(tile_env) == 1 : (!big && mid_tiles >= 192 && mid_tiles <= 256);
-    xmk::trace("fp8_gemm m=%lld n=%lld k=%lld -> %s", (long long)m, (long long)n, (long long)k,
+    xmk::trace("fp8_gemm m=%lld n=%lld k=%lld rhs_t=%d -> %s", (long long)m, (long long)n, (long long)k, rhs_transpose,
                mid ? "mfma_256x128" : big ? "mfma_256x256" : "mfma_128x128");
     if (mid) {
       p.tiles_m = (int)xmk::ceil_div(m, 256); p.tiles_n = (int)xmk::ceil_div(n, 128);
-      hipLaunchKernelGGL((fp8_gemm_kernel<256, 128, 2, 2, 4>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
+      if (fast_kn) hipLaunchKernelGGL((fp8_gemm_kernel<256, 128, 2, 2, 4, true>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
+      else hipLaunchKernelGGL((fp8_gemm_kernel<256, 128, 2, 2, 4>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
     } else if (tile_env ? atoi(tile_env) == 2 : big) {
       p.tiles_m = (int)xmk::ceil_div(m, 256); p.tiles_n = (int)xmk::ceil_div(n, 256);
-      hipLaunchKernelGGL((fp8_gemm_kernel<256, 256, 2, 4, 4>), dim3(p.tiles_m * p.tiles_n), dim3(512), 0, st, p);
+      if (fast_kn) hipLaunchKernelGGL((fp8_gemm_kernel<256, 256, 2, 4, 4, true>), dim3(p.tiles_m * p.tiles_n), dim3(512), 0, st, p);
+      else hipLaunchKernelGGL((fp8_gemm_kernel<256, 256, 2, 4, 4>), dim3(p.tiles_m * p.tiles_n), dim3(512), 0, st, p);
     } else {
       p.tiles_m = (int)xmk::ceil_div(m, 128); p.tiles_n = (int)xmk::ceil_div(n, 128);
-      hipLaunchKernelGGL((fp8_gemm_kernel<128, 128, 2, 2, 4>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
+      if (fast_kn) hipLaunchKernelGGL((fp8_gemm_kernel<128, 128, 2, 2, 4, true>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
+      else hipLaunchKernelGGL((fp8_gemm_kernel<128, 128, 2, 2, 4>), dim3(p.tiles_m * p.tiles_n), dim3(256), 0, st, p);
     }
   } else if (xmk::aligned(out, 8) && (int64_t)m * k < (int64_t)1 << 40) {
     xmk::trace("fp8_gemm m=%lld n=%lld k=%lld rhs_t=%d -> mfma_gather", (long long)m, (long long)n, (long long)k,

@@ -23,6 +23,10 @@ def _quant(oracle, shape, seed):
     (300, 515, 1027, False), (37, 52, 45, True), (2100, 2060, 200, False), (2100, 2060, 72, True),
     # about one 256 x 128 tile per CU: the third tile of the direct kernel, whole and with ragged edges
     (2048, 4096, 128, True), (1800, 4000, 144, True),
+    # [k,n]-stored B on the direct kernel (N % 16 == 0, K % 16 == 0): LDS transpose reads; the three tiles,
+    # ragged M / N / K-step edges
+    (512, 384, 1024, False), (300, 272, 208, False), (64, 16, 16, False), (4136, 4112, 208, False),
+    (2048, 4096, 128, False), (1800, 4000, 144, False),
 ])
 def test_fp8_gemm_shapes(xmk, oracle, m, n, k, rhs_t):
     a, sa = _quant(oracle, (m, k), 1)
@@ -38,23 +42,25 @@ def test_fp8_gemm_shapes(xmk, oracle, m, n, k, rhs_t):
     assert g <= 5e-3 and e <= 5e-3, (g, e)
 
 
-def test_config4_fp8_8192_sampled_rows(xmk, oracle):
-    """benchmark configuration 4: A, B [8192,8192] e4m3fn from N(0,1) with amax/448 scales, bf16 output."""
+@pytest.mark.parametrize("rhs_t", [True, False])
+def test_config4_fp8_8192_sampled_rows(xmk, oracle, rhs_t):
+    """benchmark configuration 4: A, B [8192,8192] e4m3fn from N(0,1) with amax/448 scales, bf16 output;
+    B stored [N, K] (rhs_t) or [K, N]."""
     n = 8192
     a, sa = _quant(oracle, (n, n), 11)
-    b, sb = _quant(oracle, (n, n), 12)  # stored [N, K]
+    b, sb = _quant(oracle, (n, n), 12)
     out = torch.empty((n, n), dtype=torch.bfloat16, device="cuda")
     xmk.fp8_gemm(to_dev(a, "f8"), to_dev(b, "f8"), torch.tensor([sa], device="cuda"),
-                 torch.tensor([sb], device="cuda"), out, rhs_transpose=True)
+                 torch.tensor([sb], device="cuda"), out, rhs_transpose=rhs_t)
     torch.cuda.synchronize()
     rows = np.arange(3, n, 512)
-    _, ref = oracle.fp8_gemm(a[rows], b, sa, sb, rhs_t=True)
+    _, ref = oracle.fp8_gemm(a[rows], b, sa, sb, rhs_t=rhs_t)
     g, e = oracle.rel_err(out[torch.from_numpy(rows).cuda()].float().cpu().numpy(), ref)
     print(f"config4 fp8: global {g:.2e} elementwise {e:.2e}")
     assert g <= 5e-2 and e <= 5e-2
     # identity-like property over the whole output: row sums equal A @ rowsum(B^T) (linearity)
     table = oracle.to_f32(np.arange(256, dtype=np.uint8), oracle.F8E4M3FN).astype(np.float64)
-    colsum = table[b].sum(axis=0)
+    colsum = table[b].sum(axis=0 if rhs_t else 1)
     expect = (table[a] @ colsum) * float(sa) * float(sb)
     got = out.double().sum(dim=1).cpu().numpy()
     assert np.abs(got - expect).max() <= 2e-2 * np.abs(expect).max() + 1.0
