@@ -125,7 +125,7 @@ def wl_fp8(torch, xmk, m, n, k, rhs_t=True):
     return dict(name=f"gemm_fp8_e4m3_{m}x{n}x{k}{'_rhsT' if rhs_t else '_rhs_kn'}",
                 fn=lambda: xmk.fp8_gemm(qa, qb, sa, sb, out, rhs_transpose=rhs_t),
                 flops=2.0 * m * n * k, bytes=1.0 * (m * k + k * n) + 2.0 * m * n, bound="mfma", dtype="fp8",
-                kernel="fp8_gemm_kernel" if rhs_t else "fp8_gemm_kernel")
+                kernel="fp8_gemm_kernel")
 
 
 def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
