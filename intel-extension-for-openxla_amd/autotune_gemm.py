@@ -2,6 +2,10 @@
 csrc/gemm_policy_table.h with the shapes where the heuristic's choice is not the fastest.
 
     python autotune_gemm.py [--shapes m,n,k ...] [--dry-run]
+    python autotune_gemm.py --small [--shapes m,n,k ...] [--dry-run]
+
+--small tunes the decode-sized row counts (m = 1 .. 32) of the same list over tile policy x number of K
+slices (xmk_gemm_ws with scratch; XMK_GEMM_SPLITK forces the slices) and merges the winners into the table.
 
 The counterpart of the reference's tuned table (xetla/gemm/gemm.cc:31-285) and of its
 GemmAlgorithmPicker measurement loop (gemm_impl_picker.cc:124-185).  One worker process per
@@ -12,6 +16,7 @@ import argparse
 import importlib
 import json
 import os
+import re
 import subprocess
 import sys
 
@@ -27,6 +32,12 @@ NK = [(4096, 4096), (11008, 4096), (4096, 11008), (16384, 4096), (4096, 16384), 
       (5120, 13824), (8192, 8192), (7168, 8192), (8192, 7168), (14336, 7168), (7168, 14336), (12288, 4096)]
 MS = [64, 128, 256, 512, 1024, 2048, 4096]
 DEFAULT_SHAPES = [(m, n, k) for m in MS for (n, k) in NK] + [(8192, 8192, 8192)]
+# Decode-sized shapes: the m = 1, 4, 32 rows of gemm.cc:33-47 and the row counts between, on the GPT-J
+# projections (4096 x 4096, 4096 -> 16384, 16384 -> 4096, the stacked q/k/v 4096 -> 12288).
+SMALL_NK = [(4096, 16384), (16384, 4096), (4096, 4096), (12288, 4096)]
+SMALL_MS = [1, 4, 8, 16, 32]
+SMALL_SHAPES = [(m, n, k) for m in SMALL_MS for (n, k) in SMALL_NK]
+SPLITS = [1, 2, 4, 8, 16]
 
 
 TILE_RATE = [1.0, 0.75, 0.60, 0.55, 0.90]
@@ -42,6 +53,95 @@ def heuristic(m, n, k):
         if score > best_score:
             best, best_score = i, score
     return best
+
+
+def worker_small(shapes):
+    """Times xmk_gemm_ws (scratch for up to 16 slices) from a HIP graph of 20 launches per replay."""
+    sys.path.insert(0, os.path.dirname(HERE))
+    import torch
+    xmk = importlib.import_module(os.path.basename(HERE))
+    out = {}
+    for (m, n, k) in shapes:
+        a = (torch.randn((m, k), device="cuda") * k ** -0.5).bfloat16()
+        bs = [(torch.randn((k, n), device="cuda") * k ** -0.5).bfloat16() for _ in range(4)]  # rotate past the cache
+        c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        ws = torch.empty((16 * m * n,), dtype=torch.float32, device="cuda")
+        st = torch.cuda.Stream()
+        with torch.cuda.stream(st):
+            for b in bs:
+                xmk.run_gemm(a, b, c, workspace=ws)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=st):
+                for i in range(20):
+                    xmk.run_gemm(a, bs[i % 4], c, workspace=ws)
+        torch.cuda.synchronize()
+        g.replay()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best = 1e30
+        for _ in range(5):
+            s.record()
+            g.replay()
+            e.record()
+            torch.cuda.synchronize()
+            best = min(best, s.elapsed_time(e) / 20)
+        out[f"{m},{n},{k}"] = best
+    print("RESULT " + json.dumps(out), flush=True)
+
+
+def run_worker(shapes, env_extra, flag):
+    env = dict(os.environ, **env_extra)
+    cmd = [sys.executable, os.path.abspath(__file__), flag, "--shapes"] + [f"{m},{n},{k}" for m, n, k in shapes]
+    r = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=900)
+    line = [l for l in r.stdout.splitlines() if l.startswith("RESULT ")]
+    if r.returncode != 0 or not line:
+        sys.exit(f"worker {env_extra} failed:\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}")
+    return json.loads(line[0][7:])
+
+
+def load_table():
+    """(m, n, k) -> (policy, ksplit, comment) of the table as it stands."""
+    rows = {}
+    if os.path.exists(TABLE):
+        for l in open(TABLE):
+            m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+)\},\s*//\s*(.*)", l)
+            if m and int(m.group(1)) > 0:
+                rows[(int(m.group(1)), int(m.group(2)), int(m.group(3)))] = (int(m.group(4)), int(m.group(5)), m.group(6))
+    return rows
+
+
+def write_table(rows):
+    with open(TABLE, "w") as f:
+        f.write("// Tuned (m, n, k) -> {policy index, K slices} table.  GENERATED by autotune_gemm.py; do not edit by hand.\n")
+        f.write("// Shapes where a choice other than the heuristic's was measured faster on an MI355X (bf16, row-major\n")
+        f.write("// operands).  K slices 0: tile policy only (TFLOP/s heuristic -> chosen); K slices >= 1: the number of\n")
+        f.write("// slices and their tile for xmk_gemm_ws (microseconds default -> chosen).\n")
+        f.write("constexpr TunedShape kTunedShapes[] = {\n")
+        for (m, n, k) in sorted(rows):
+            pol, ks, note = rows[(m, n, k)]
+            f.write(f"    {{{m}, {n}, {k}, {pol}, {ks}}},  // {note}\n")
+        f.write("    {0, 0, 0, 0, 0},\n};\n")
+    print(f"wrote {TABLE}: {len(rows)} shapes")
+
+
+def tune_small(shapes, args):
+    base = run_worker(shapes, {}, "--worker-small")
+    print("default choice measured", flush=True)
+    cand = {}
+    for pol in range(len(POLICIES)):
+        for ks in SPLITS:
+            cand[(pol, ks)] = run_worker(shapes, {"XMK_GEMM_POLICY": str(pol), "XMK_GEMM_SPLITK": str(ks)}, "--worker-small")
+            print(f"policy {pol} x {ks} slices measured", flush=True)
+    rows = load_table()
+    for (m, n, k) in shapes:
+        key = f"{m},{n},{k}"
+        best = min(cand, key=lambda c: cand[c][key])
+        t0, t1 = base[key] * 1e3, cand[best][key] * 1e3
+        print(f"{key:>18}: default {t0:7.2f} us  best {t1:7.2f} us  = {POLICIES[best[0]]} x {best[1]} slices")
+        rows.pop((m, n, k), None)
+        if t1 < t0 * (1.0 - args.margin):
+            rows[(m, n, k)] = (best[0], best[1], f"{t0:.1f} -> {t1:.1f} us")
+    if not args.dry_run:
+        write_table(rows)
 
 
 def worker(shapes):
@@ -73,22 +173,25 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--shapes", nargs="*", help="m,n,k triples (default: the built-in LLM shape list)")
     ap.add_argument("--worker", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--worker-small", action="store_true", help=argparse.SUPPRESS)
+    ap.add_argument("--small", action="store_true", help="tune m = 1 .. 32 over tile policy x K slices")
     ap.add_argument("--dry-run", action="store_true", help="measure and print, do not write the table")
     ap.add_argument("--margin", type=float, default=0.03, help="ignore wins smaller than this fraction")
     args = ap.parse_args()
-    shapes = [tuple(int(x) for x in s.split(",")) for s in args.shapes] if args.shapes else DEFAULT_SHAPES
+    default = SMALL_SHAPES if (args.small or args.worker_small) else DEFAULT_SHAPES
+    shapes = [tuple(int(x) for x in s.split(",")) for s in args.shapes] if args.shapes else default
     if args.worker:
         worker(shapes)
         return
+    if args.worker_small:
+        worker_small(shapes)
+        return
+    if args.small:
+        tune_small(shapes, args)
+        return
     times = []
     for pol in range(len(POLICIES)):
-        env = dict(os.environ, XMK_GEMM_POLICY=str(pol))
-        cmd = [sys.executable, os.path.abspath(__file__), "--worker", "--shapes"] + [f"{m},{n},{k}" for m, n, k in shapes]
-        r = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=900)
-        line = [l for l in r.stdout.splitlines() if l.startswith("RESULT ")]
-        if r.returncode != 0 or not line:
-            sys.exit(f"worker for policy {pol} failed:\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}")
-        times.append(json.loads(line[0][7:]))
+        times.append(run_worker(shapes, {"XMK_GEMM_POLICY": str(pol)}, "--worker"))
         print(f"policy {pol} ({POLICIES[pol]}) measured", flush=True)
     rows = []
     for (m, n, k) in shapes:
@@ -101,15 +204,10 @@ def main():
             rows.append((m, n, k, best, tf[h], tf[best]))
     if args.dry_run:
         return
-    with open(TABLE, "w") as f:
-        f.write("// Tuned (m, n, k) -> policy index table.  GENERATED by autotune_gemm.py; do not edit by hand.\n")
-        f.write("// Shapes where a policy other than the heuristic's was measured faster on an MI355X\n")
-        f.write("// (bf16, row-major operands); the comment gives TFLOP/s heuristic -> chosen.\n")
-        f.write("constexpr TunedShape kTunedShapes[] = {\n")
-        for (m, n, k, best, a, b) in rows:
-            f.write(f"    {{{m}, {n}, {k}, {best}}},  // {a:.0f} -> {b:.0f}\n")
-        f.write("    {0, 0, 0, 0},\n};\n")
-    print(f"wrote {TABLE}: {len(rows)} shapes")
+    table = {key: v for key, v in load_table().items() if v[1] != 0 or key not in set(shapes)}
+    for (m, n, k, best, a, b) in rows:
+        table[(m, n, k)] = (best, 0, f"{a:.0f} -> {b:.0f}")
+    write_table(table)
 
 
 if __name__ == "__main__":

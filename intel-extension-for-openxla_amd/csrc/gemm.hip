@@ -203,13 +203,27 @@ extern "C" const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int
 
 namespace {
 // out1 / out2: further outputs of the shared-lhs three-GEMM form, or null for a plain GEMM.
-int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream);
+// policy: tile policy to use instead of select_policy's choice (the K-split planner's), or -1.
+int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int policy = -1);
 
 // K slices worth using for a plain 16-bit GEMM of this shape when scratch is available: few
 // output tiles (the device has 256 CUs) and a long reduction.  1: do not split.
-int plan_splitk(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k) {
+// *policy: the tile policy of the slices (-1: whatever select_policy picks for a slice).
+int plan_splitk(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k, int* policy) {
+  *policy = -1;
   if (d->batch_size != 1 || n % 4 != 0) return 1;
   if (d->dtype_in != XMK_BF16 && d->dtype_in != XMK_F16) return 1;
+  auto divides = [&](int ks) { return ks >= 1 && ks <= 16 && k % (ks * 8) == 0; };
+  // XMK_GEMM_SPLITK=<slices> overrides the choice (read once; the autotuner's handle).
+  static const int forced = [] {
+    const char* e = getenv("XMK_GEMM_SPLITK");
+    return e ? atoi(e) : 0;
+  }();
+  if (forced >= 1) return divides(forced) ? forced : 1;
+  if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit >= 1 && divides(t->ksplit)) {
+    if (t->ksplit > 1) *policy = t->policy;
+    return t->ksplit;
+  }
   const Policy& pol = kPolicies[select_policy(m, n, k)];
   const int64_t tiles = xmk::ceil_div(m, pol.bm) * xmk::ceil_div(n, pol.bn);
   int ks = 1;
@@ -235,7 +249,8 @@ extern "C" size_t xmk_gemm_workspace_bytes(const xmk_gemm_desc* d) {
   int64_t m, n, k;
   gemm_dims(d, &m, &n, &k);
   if (m <= 0 || n <= 0 || k <= 0) return 0;
-  const int ks = plan_splitk(d, m, n, k);
+  int pol;
+  const int ks = plan_splitk(d, m, n, k, &pol);
   return ks > 1 ? (size_t)ks * m * n * sizeof(float) : 0;
 }
 
@@ -246,7 +261,8 @@ extern "C" int xmk_gemm_ws(const xmk_gemm_desc* d, void* workspace, size_t works
     return run_gemm(d, nullptr, nullptr, stream);
   int64_t m, n, k;
   gemm_dims(d, &m, &n, &k);
-  const int ks = plan_splitk(d, m, n, k);
+  int slice_policy;
+  const int ks = plan_splitk(d, m, n, k, &slice_policy);
   // Pass 1: the K slices as a batched GEMM into fp32 partial sums (no epilogue); a slice is a
   // column range of lhs and a row (or column) range of rhs, so only the batch strides change.
   xmk_gemm_desc p = *d;
@@ -281,7 +297,7 @@ extern "C" int xmk_gemm_ws(const xmk_gemm_desc* d, void* workspace, size_t works
       (d->dtype_out != d->dtype_in && d->dtype_out != XMK_F32))
     return run_gemm(d, nullptr, nullptr, stream);  // reports the error
   xmk::trace("gemm m=%lld n=%lld k=%lld -> split K %d ways", (long long)m, (long long)n, (long long)k, ks);
-  int rc = run_gemm(&p, nullptr, nullptr, stream);
+  int rc = run_gemm(&p, nullptr, nullptr, stream, slice_policy);
   if (rc != XMK_OK) return rc;
   ReduceParams r;
   r.partial = (const float*)workspace; r.out = d->out.data; r.c = d->beta != 0.0f ? d->c : nullptr;
@@ -305,7 +321,7 @@ extern "C" int xmk_gemm_qkv(const xmk_gemm_desc* d, void* out_k, void* out_v, vo
 }
 
 namespace {
-int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
+int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int policy) {
   if (!d) return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: null descriptor");
   if (!d->lhs.data || !d->rhs.data || !d->out.data)
     return xmk::fail(XMK_INVALID_ARGUMENT, "gemm: null operand");
@@ -405,7 +421,7 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream) {
     const bool a_mc = lhs.transpose != 0;   // stored [K, M]
     const bool b_mc = rhs.transpose == 0;   // stored [K, N]
     const int batch = qkv ? 3 : (int)d->batch_size;
-    const int pol = select_policy(m, n, k, batch);
+    const int pol = (policy >= 0 && policy < kNumPolicies) ? policy : select_policy(m, n, k, batch);
     xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s",
                (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
                rhs.transpose, d->epilogue, d->beta, gather ? kGatherPolicy.name : kPolicies[pol].name);

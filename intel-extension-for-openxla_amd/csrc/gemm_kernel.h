@@ -652,10 +652,17 @@ constexpr int kNumPolicies = sizeof(kPolicies) / sizeof(kPolicies[0]);
 // (gemm_policy_table.h, written by autotune_gemm.py from measurements) take the policy
 // recorded there, as the reference's configMap does (gemm.cc:31-285).
 // XMK_GEMM_POLICY=<index> forces one policy for every shape (what the autotuner uses).
+// ksplit: K slices to use when the caller supplies scratch (xmk_gemm_ws); 0 = no tuned value, the
+// planner's own rule decides.  With ksplit > 1 `policy` is the tile of the slices.
 struct TunedShape {
-  int m, n, k, policy;
+  int m, n, k, policy, ksplit;
 };
 #include "gemm_policy_table.h"
+inline const TunedShape* tuned_shape(int64_t m, int64_t n, int64_t k) {
+  for (const TunedShape& t : kTunedShapes)
+    if (t.m == m && t.n == n && t.k == k) return &t;
+  return nullptr;
+}
 inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1) {
   static const int forced = [] {
     const char* e = getenv("XMK_GEMM_POLICY");
@@ -664,8 +671,7 @@ inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1) {
   }();
   if (forced >= 0) return forced;
   if (batch == 1)
-    for (const TunedShape& t : kTunedShapes)
-      if (t.m == m && t.n == n && t.k == k) return t.policy;
+    if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit <= 1) return t->policy;
   // Heuristic: the policy with the best estimated throughput = (what the tile sustains when the
   // device is full) x (share of the 256 CUs busy over the tile waves) x (share of the tiles' area
   // inside the matrix).  The per-tile figures are measured large-shape rates relative to 256x256.
