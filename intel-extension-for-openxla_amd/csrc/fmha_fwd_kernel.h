@@ -11,16 +11,16 @@
 //   O^T += V^T P^T : P stays in registers (the S accumulator registers, converted, ARE the B
 //                 operand); V is staged untransposed [key][h] and read with the LDS transpose
 //                 loads, which deliver four consecutive keys of one h.
-// K and V tiles go from global memory straight into LDS (buffer_load ... lds), two stages each,
-// the loads of the next tiles in flight while the current ones are computed.
+// K and V half tiles go from global memory straight into LDS (buffer_load ... lds), a ring of four
+// stages each, the loads of the next three half tiles in flight while the current one is computed.
 //
 // The loop is a three-stage software pipeline over half tiles h (32 keys): in one step the matrix
 // cores run the P V product of half tile h-1 and the S product of half tile h+1 while the vector
 // ALU turns S_h into P_h (row max, exponentials, rounding, row sums).  The matrix instructions of
-// a step depend on no vector result of the same step, and a step is one basic block, so the
-// instruction scheduler can deal them evenly among the vector instructions: an 8-pass matrix
-// instruction leaves about seven vector issue slots, which is what the softmax of its share of
-// the scores needs.
+// a step depend on no vector result of the same step.  The step is written out as one slot per
+// matrix instruction (its LDS fragment reads a few slots ahead, a fixed share of the vector work),
+// the slots separated by scheduling fences: an 8-pass matrix instruction leaves about seven vector
+// issue slots, which is what the softmax of its share of the scores needs.
 //
 // Online softmax in the exp2 domain: the scale is folded into the exponent (one FMA per
 // element), the running reference max only moves when a row max exceeds it by more than
