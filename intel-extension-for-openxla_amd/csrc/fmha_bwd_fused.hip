@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
   constexpr int NW = 4;
   constexpr int ROWB = HP * 2;               // bytes of one tile row in LDS
   constexpr int CPR = ROWB / 16;             // 16-byte chunks per row
-  constexpr int KMASK = CPR >= 16 ? 15 : 7;  // chunk ^= row & KMASK
+  constexpr int KMASK = 15;                  // the swizzle repeats every KMASK + 1 rows
   constexpr int TILE = BS * ROWB;
   constexpr int RPL = 1024 / ROWB;           // tile rows per 1 KiB load
   constexpr int NL = TILE / 1024 / NW;       // loads per wave per tile
@@ -122,6 +122,16 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g = lane >> 5, l32 = lane & 31;
+  // A tile row stores its 16-byte chunk c at position c ^ swz(row).  One tile serves two kinds of reads: row
+  // fragments (16 lanes = 16 consecutive rows, one chunk column: swz must differ among 16 consecutive rows)
+  // and transposed fragments (32 lanes = 4 consecutive rows x 4 adjacent chunks: bits 2-3 of swz must differ
+  // among 4 consecutive rows, or the four rows land on the same banks).  Rows of 256 bytes and more: the two
+  // bit pairs of row & 15, exchanged.  Rows of 128 bytes (8 chunks, two rows per 256 bytes of banks): the row's
+  // parity already separates neighbours, and bits 1..3 of the row are dealt so that rows r and r + 2 differ in
+  // bit 2 of swz and rows r and r + 8 in bit 1.
+  auto swz = [](int row) {
+    return CPR >= 16 ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+  };
   // Each XCD (own L2) gets a contiguous range of (unit, owner block) pairs: the owner blocks of a
   // unit stream the same tiles.
   const int wg = (int)(blockIdx.x % 8) * p.per_xcd + (int)(blockIdx.x / 8);
@@ -173,13 +183,13 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
 
   // ---- streamed tile loads, global -> LDS, as in the forward kernel: load j = i * NW + wave fills
   // LDS bytes [1024 j, +1024) of the tile; lane l lands at row j * RPL + l / CPR, chunk l % CPR, and
-  // fetches the global chunk that belongs there under the swizzle chunk ^= row & KMASK.
+  // fetches the global chunk that belongs there under the swizzle (swz below).
   const int lrow = wave * RPL + lane / CPR;
   uint32_t koff[KV];
 #pragma unroll
   for (int v = 0; v < KV; ++v) {
     const int row = lrow + v * LROWS;
-    const int chunk = (lane % CPR) ^ (row & KMASK);
+    const int chunk = (lane % CPR) ^ swz(row);
     koff[v] = chunk * 8 < H ? (uint32_t)((lrow * H + chunk * 8) * 2) : kOob;
   }
   const uint32_t lstride = (uint32_t)(LROWS * H * 2);
@@ -207,7 +217,7 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
   // Row fragment (kt, s): tile row 32 kt + l%32, logical chunk 2 s + g.
   int kbase[KS];
 #pragma unroll
-  for (int s = 0; s < KS; ++s) kbase[s] = l32 * ROWB + (((2 * s + g) ^ (l32 & KMASK)) << 4);
+  for (int s = 0; s < KS; ++s) kbase[s] = l32 * ROWB + (((2 * s + g) ^ swz(l32)) << 4);
   // Transposed fragment (group u, h tile ht): two transpose reads; within a 16-lane block lane pl
   // addresses tile row 16 u + 4 g + pl/4 (+8 for the second read), h = cb + 4 (pl%4) .. +3.
   int tbase[HT][2];
@@ -219,8 +229,8 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
       const int chunk = col >> 3, within = (col & 7) * 2;
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2) {
-        const int row = 4 * g + (pl >> 2) + 8 * h2;  // + 16 u: does not change row & KMASK
-        tbase[ht][h2] = row * ROWB + ((chunk ^ (row & KMASK)) << 4) + within;
+        const int row = 4 * g + (pl >> 2) + 8 * h2;  // + 16 u: does not change swz(row)
+        tbase[ht][h2] = row * ROWB + ((chunk ^ swz(row)) << 4) + within;
       }
     }
   }
