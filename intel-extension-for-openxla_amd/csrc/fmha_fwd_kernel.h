@@ -152,7 +152,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   constexpr int BR = NW * 32;                // query rows per work-group
   constexpr int ROWB = HP * 2;               // bytes of one K / V row in LDS
   constexpr int CPR = ROWB / 16;             // 16-byte chunks per row
-  constexpr int KMASK = CPR >= 16 ? 15 : 7;  // K rows: chunk ^= key & KMASK (16 lanes -> 16 bank groups)
+  constexpr int KMASK = 15;                  // the K swizzle repeats every KMASK + 1 rows
   constexpr int HALF = 32 * ROWB;            // one K or V half tile (32 keys): one LDS stage
   constexpr int NST = 4;                     // stages of the K ring and of the V ring
   constexpr int RPL = 1024 / ROWB;           // tile rows per 1 KiB load
@@ -212,12 +212,16 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   // ---- K / V half-tile loads, global -> LDS.  Load j = i * NW + wave fills LDS bytes [1024 j, +1024)
   // of the stage, i.e. half-tile rows j * RPL ..; lane l lands at row j * RPL + l / CPR, chunk l % CPR,
   // and fetches the global chunk that belongs there under the stage's swizzle.
+  // K rows: chunk ^= kswz(key), so that the 16 lanes of a fragment read (16 consecutive keys, one chunk column)
+  // touch 16 different bank groups: with 128-byte rows two keys share 256 bytes of banks and the key's parity
+  // already separates them.
+  auto kswz = [](int key) { return CPR >= 16 ? (key & 15) : ((key >> 1) & 7); };
   const int lrow = wave * RPL + lane / CPR;  // half-tile row of this lane in load 0; load i: + i * LROWS
   uint32_t koff[KV];
 #pragma unroll
   for (int v = 0; v < KV; ++v) {
     const int row = lrow + v * LROWS;
-    const int chunk = (lane % CPR) ^ (row & KMASK);
+    const int chunk = (lane % CPR) ^ kswz(row);
     koff[v] = chunk * 8 < H ? (uint32_t)((lrow * H + chunk * 8) * 2) : kOob;
   }
   // V rows: chunk ^= vswz(key).  A transpose read touches 4 chunks of each of 4 consecutive keys;
@@ -245,7 +249,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   // K fragment (step s): key row l%32 of the half tile, logical chunk 2 s + g.
   int kbase[KS];
 #pragma unroll
-  for (int s = 0; s < KS; ++s) kbase[s] = l32 * ROWB + (((2 * s + g) ^ (l32 & KMASK)) << 4);
+  for (int s = 0; s < KS; ++s) kbase[s] = l32 * ROWB + (((2 * s + g) ^ kswz(l32)) << 4);
   // V^T fragment (key group u of the half tile, h tile ht): two transpose reads; within a 16-lane block
   // lane pl addresses key row 16 u + 4 g + pl/4 (+8 for the second read), h = cb + 4 (pl%4) .. +3.
   int vbase[HT][2];

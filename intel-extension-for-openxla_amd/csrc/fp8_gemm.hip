@@ -61,7 +61,7 @@ struct Fp8Frag {
 };
 
 // The same fragments from a tile stored [64 k][BN columns] (row = BN bytes, 16-byte chunks XOR-swizzled
-// by the loader with swz<true, BN / 2, 64>(k)).  ds_read_b64_tr_b8 works on blocks of 16 lanes: lane p
+// by the loader with swz<true, BN / 2, 64, 1>(k)).  ds_read_b64_tr_b8 works on blocks of 16 lanes: lane p
 // of a block addresses row kb + p / 2, bytes cb + 8 (p % 2) .. +7 and receives column cb + p, rows
 // kb .. kb + 7.  Blocks 0 and 1 of the wave cover columns 0..15 and 16..31 of the slab for k half 0,
 // blocks 2 and 3 the same columns for k half 1; four reads, 8 rows apart, give a lane its 32 k.  The
@@ -75,7 +75,7 @@ struct Fp8FragKN {
 #pragma unroll
     for (int t = 0; t < T; ++t) {
       const int col = col0 + t * 32 + ((lane >> 4) & 1) * 16 + 8 * (p & 1);
-      base[t] = k * BN + (((col >> 4) ^ gemm_impl::swz<true, BN / 2, 64>(k)) << 4) + (col & 15);
+      base[t] = k * BN + (((col >> 4) ^ gemm_impl::swz<true, BN / 2, 64, 1>(k)) << 4) + (col & 15);
     }
   }
   // t counts 32-column slabs from col0; only slabs this wave owns are read.
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
   // The loader works in 2-byte units: BK = 32 units = 64 bytes.
   typedef gemm_impl::Loader<false, BM, 32, NWAVES> LoaderA;
   // B [n,k]: BN rows of 64 bytes; B [k,n]: 64 rows of BN bytes (BN / 2 two-byte units).
-  typedef std::conditional_t<BKN, gemm_impl::Loader<true, BN / 2, 64, NWAVES>, gemm_impl::Loader<false, BN, 32, NWAVES>>
+  typedef std::conditional_t<BKN, gemm_impl::Loader<true, BN / 2, 64, NWAVES, 1>, gemm_impl::Loader<false, BN, 32, NWAVES>>
       LoaderB;
   constexpr int LOADS = LoaderA::NL + LoaderB::NL;  // per wave per K step
   static_assert(NSTAGE >= 3, "the barrier leaves the running step's loads in flight");

@@ -103,15 +103,22 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base) {
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
-// XOR applied to the 16-byte chunk index inside an LDS row, chosen so that the 16 lanes the
-// LDS serves per cycle (256 bytes) touch 16 different 16-byte bank groups.
-//   KC, BK = 64: rows of 128 bytes (8 chunks); KC, BK = 32: rows of 64 bytes (4 chunks).
-//   MC: rows of ROWS * 2 bytes; the XOR is even so that 32-byte pairs stay together.
-template <bool MC, int ROWS, int BK>
+// XOR applied to the 16-byte chunk index inside an LDS row, chosen so that the lanes the LDS serves
+// together touch different banks (256 bytes of banks).
+//   KC, BK = 64: rows of 128 bytes (8 chunks); KC, BK = 32: rows of 64 bytes (4 chunks); read with
+//       ds_read_b128, 16 lanes = 16 rows of one chunk column.
+//   MC: rows of ROWS * 2 bytes, read with the LDS transpose loads.  16-bit elements (EB = 2,
+//       ds_read_b64_tr_b16): 32 lanes take 64 bytes of each of 4 consecutive k rows, so rows of 256 bytes and
+//       more move by whole 64-byte groups, (k & 3) << 2; with 128-byte rows two rows share the banks and
+//       (k & 3) << 1 separates the four.  8-bit elements (EB = 1, ds_read_b64_tr_b8): 32 lanes take 32 bytes of
+//       each of 8 consecutive k rows, (k & 7) << 1 (rows of 256 bytes and more).  The XOR is even so that 32-byte pairs
+//       stay together.
+template <bool MC, int ROWS, int BK, int EB = 2>
 __device__ __forceinline__ int swz(int row_or_k) {
   if constexpr (!MC) return BK == 64 ? (row_or_k & 7) : ((row_or_k >> 2) & 3);
-  else if constexpr (ROWS >= 128) return (row_or_k & 7) << 1;
-  else return (row_or_k & 3) << 1;
+  else if constexpr (ROWS < 128) return (row_or_k & 3) << 1;  // 8 chunks per row: the XOR stays below 8
+  else if constexpr (EB == 1) return (row_or_k & 7) << 1;
+  else return (row_or_k & 3) << 2;
 }
 
 // One operand tile = BK k x ROWS rows/cols = ROWS * BK * 2 bytes of LDS in both layouts.
@@ -120,7 +127,7 @@ __device__ __forceinline__ int swz(int row_or_k) {
 // chunk column in every load: its global byte offset is voff + i * sstride, with voff in one
 // VGPR and the per-load part in the instruction's scalar offset.  Row/column validity is
 // kept as one lane mask per load (scalar registers).
-template <bool MC, int ROWS, int BK, int NWAVES>
+template <bool MC, int ROWS, int BK, int NWAVES, int EB = 2>
 struct Loader {
   static constexpr int RB = MC ? ROWS * 2 : BK * 2;  // LDS row, bytes
   static constexpr int CPR = RB / 16;                // chunks per LDS row
@@ -137,7 +144,7 @@ struct Loader {
 
   __device__ __forceinline__ void init(int64_t ld, int valid, int wave, int lane) {
     const int lrow = wave * RPL + lane / CPR;  // LDS row in load 0: operand row (KC) or k (MC)
-    const int chunk = (lane % CPR) ^ swz<MC, ROWS, BK>(lrow);
+    const int chunk = (lane % CPR) ^ swz<MC, ROWS, BK, EB>(lrow);
     voff = (uint32_t)(((int64_t)lrow * ld + chunk * 8) * 2);
     sstride = (uint32_t)(LSTRIDE * ld * 2);
     if constexpr (!MC) {
@@ -184,7 +191,7 @@ struct Loader {
   __device__ __forceinline__ u32x4 gather_load(int i, const uint16_t* base, int64_t ld, int valid, int kleft,
                                                int wave, int lane, int vec) const {
     const int lrow = wave * RPL + lane / CPR + i * LSTRIDE;                       // LSTRIDE % 8 == 0:
-    const int c0 = ((lane % CPR) ^ swz<MC, ROWS, BK>(wave * RPL + lane / CPR)) * 8;  // same swizzle for every i
+    const int c0 = ((lane % CPR) ^ swz<MC, ROWS, BK, EB>(wave * RPL + lane / CPR)) * 8;  // same swizzle for every i
     const int row = MC ? c0 : lrow;   // operand row / column of element 0
     const int k = MC ? lrow : c0;     // k (inside the K step) of element 0
     const uint16_t* src = MC ? base + (int64_t)k * ld + row : base + (int64_t)row * ld + k;
