@@ -106,7 +106,8 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr;
 // XOR applied to the 16-byte chunk index inside an LDS row, chosen so that the lanes the LDS serves
 // together touch different banks (256 bytes of banks).
 //   KC, BK = 64: rows of 128 bytes (8 chunks); KC, BK = 32: rows of 64 bytes (4 chunks); read with
-//       ds_read_b128, 16 lanes = 16 rows of one chunk column.
+//       ds_read_b128, 16 lanes = 16 rows of one chunk column.  Two (four) rows share 256 bytes of banks and
+//       are apart by their position there, so the XOR counts pairs (quadruples) of rows.
 //   MC: rows of ROWS * 2 bytes, read with the LDS transpose loads.  16-bit elements (EB = 2,
 //       ds_read_b64_tr_b16): 32 lanes take 64 bytes of each of 4 consecutive k rows, so rows of 256 bytes and
 //       more move by whole 64-byte groups, (k & 3) << 2; with 128-byte rows two rows share the banks and
@@ -115,7 +116,7 @@ typedef __attribute__((address_space(3))) void* lds_void_ptr;
 //       stay together.
 template <bool MC, int ROWS, int BK, int EB = 2>
 __device__ __forceinline__ int swz(int row_or_k) {
-  if constexpr (!MC) return BK == 64 ? (row_or_k & 7) : ((row_or_k >> 2) & 3);
+  if constexpr (!MC) return BK == 64 ? ((row_or_k >> 1) & 7) : ((row_or_k >> 2) & 3);
   else if constexpr (ROWS < 128) return (row_or_k & 3) << 1;  // 8 chunks per row: the XOR stays below 8
   else if constexpr (EB == 1) return (row_or_k & 7) << 1;
   else return (row_or_k & 3) << 2;
@@ -135,7 +136,7 @@ struct Loader {
   static constexpr int NL = ROWS * BK * 2 / 1024 / NWAVES;
   static constexpr int LSTRIDE = NWAVES * RPL;       // LDS rows between consecutive loads of a wave
   static_assert(NL >= 1, "tile too small for this many waves");
-  static_assert(LSTRIDE % 8 == 0, "swizzle must repeat from load to load");
+  static_assert(LSTRIDE % 16 == 0 || (LSTRIDE % 8 == 0 && (MC || BK == 32)), "swizzle must repeat from load to load");
   uint32_t voff;     // byte offset of this lane's chunk in load 0, from the tile origin
   uint32_t sstride;  // bytes between consecutive loads of this wave (uniform)
   int kin0;          // k (inside the K step) of this lane's chunk in load 0
