@@ -295,6 +295,15 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
         st[kt] = Elem<T>::mfma(__builtin_bit_cast(V8, kv), of[s], st[kt]);
       }
   };
+  // The same for the 32 streamed rows of half kt alone.
+  auto scores_half = [&](const char* __restrict__ tile, const V8 (&of)[KS], int kt, floatx16& st) {
+    st = zero16();
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const u32x4 kv = *reinterpret_cast<const u32x4*>(tile + kbase[s] + kt * 32 * ROWB);
+      st = Elem<T>::mfma(__builtin_bit_cast(V8, kv), of[s], st);
+    }
+  };
   // acc^T += Stream_tile^T . F, with F given as four B-operand fragments (group u contracts the
   // streamed rows 16 u + {0..3, 8..11} + 4 g).
   auto accumulate = [&](const char* __restrict__ tile, const V8 (&fr)[4], floatx16 (&acc)[HT]) {
@@ -330,18 +339,24 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
     }
     float bs[BIAS ? 2 : 1][16];
     if constexpr (BIAS) load_bias(t0, bs);
+    // The dK launch of the larger head sizes holds both owner operands, the accumulators and the scores of
+    // a whole block only with spills (30 registers): it goes through the block's two halves one after the
+    // other, so that one half's scores are dead before the other's are made.
+    constexpr bool BY_HALF = OWNER_K && DS && !PV && HP >= 128;
     floatx16 sc[2], dp[2];
-    scores(c1, of1, sc);
-    if constexpr (DS) scores(c2, of2, dp);
+    if constexpr (!BY_HALF) {
+      scores(c1, of1, sc);
+      if constexpr (DS) scores(c2, of2, dp);
+    }
     // sc[kt][i], dp[kt][i] <-> streamed row t0 + 32 kt + 8 (i/4) + 4 g + i%4, owner row `orow`.
     V8 pf[4], df[4];
     // Blocks that end inside the streamed range and (causal) lie wholly on the visible side of the
     // diagonal for every row of this wave need no mask (wave-uniform test).
     const bool masked = t0 + BS > n_str || (CAUSAL && (OWNER_K ? wo0 + 31 > t0 : t0 + BS - 1 > wo0));
-    auto elementwise = [&](auto MASKED_T) {
+    auto elementwise = [&](auto MASKED_T, auto KT_LO, auto KT_HI) {
       constexpr bool MASKED = decltype(MASKED_T)::value;
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+      for (int kt = decltype(KT_LO)::value; kt < decltype(KT_HI)::value; ++kt)
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
           floatx4 l2, dd;
@@ -371,8 +386,22 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
           }
         }
     };
-    if (masked) elementwise(std::true_type{});
-    else elementwise(std::false_type{});
+    typedef std::integral_constant<int, 0> i0;
+    typedef std::integral_constant<int, 1> i1;
+    typedef std::integral_constant<int, 2> i2;
+    if constexpr (BY_HALF) {
+      scores_half(c1, of1, 0, sc[0]);
+      scores_half(c2, of2, 0, dp[0]);
+      if (masked) elementwise(std::true_type{}, i0{}, i1{});
+      else elementwise(std::false_type{}, i0{}, i1{});
+      scores_half(c1, of1, 1, sc[1]);
+      scores_half(c2, of2, 1, dp[1]);
+      if (masked) elementwise(std::true_type{}, i1{}, i2{});
+      else elementwise(std::false_type{}, i1{}, i2{});
+    } else {
+      if (masked) elementwise(std::true_type{}, i0{}, i2{});
+      else elementwise(std::false_type{}, i0{}, i2{});
+    }
     if constexpr (DS) accumulate(c1, df, acc1);
     if constexpr (PV) accumulate(c2, pf, acc2);
     // The next block's tiles have landed (this wave's loads; every wave's after the barrier), and
