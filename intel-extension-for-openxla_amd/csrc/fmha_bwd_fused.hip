@@ -369,17 +369,18 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
             const int i = 4 * qd + e;
             const float lse2 = OWNER_K ? l2[e] * kLog2e : own_lse2;
             const float dq = OWNER_K ? dd[e] : own_d;
-            float pr;
-            if constexpr (BIAS)
-              pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, __builtin_fmaf(bs[kt][i], kLog2e, -lse2)));
-            else
-              pr = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[kt][i], scale2, -lse2));
+            float arg;
+            if constexpr (BIAS) arg = __builtin_fmaf(sc[kt][i], scale2, __builtin_fmaf(bs[kt][i], kLog2e, -lse2));
+            else arg = __builtin_fmaf(sc[kt][i], scale2, -lse2);
             if constexpr (MASKED) {
+              // The mask goes into the exponent (a select on a ready value, exp2(-inf) = 0): with `pr = 0` after
+              // the exponential the compiler branches around every single exponential instead.
               const int srow = t0 + 32 * kt + 8 * qd + 4 * g + e;
               const int q = OWNER_K ? srow : orow;
               const int key = OWNER_K ? orow : srow;
-              if (srow >= n_str || (CAUSAL && key > q)) pr = 0.f;
+              arg = (srow >= n_str || (CAUSAL && key > q)) ? -INFINITY : arg;
             }
+            const float pr = __builtin_amdgcn_exp2f(arg);
             // fragment u = 2 kt + (qd >> 1) holds registers 8 (u & 1) .. +7 of tile kt
             if constexpr (PV) pf[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)pr;
             if constexpr (DS) df[2 * kt + (qd >> 1)][4 * (qd & 1) + e] = (T)(pr * (dp[kt][i] - dq));
