@@ -23,9 +23,12 @@ constexpr size_t kChunkBytes = (size_t)1 << 30;  // score-sized intermediates pe
 
 // D[row] = sum_h O[row][h] dO[row][h].  H % 8 == 0: a lane reads 8 elements (16 bytes) of each tensor;
 // LPR lanes (a power of two >= H / 8) share a row and a wave covers 64 / LPR rows.
+// With lse2 != NULL it also writes lse2[row] = lse[row] * log2(e), the form the fused kernels use in their
+// exponentials (one multiplication per row here instead of one per score there).
 template <typename T, int LPR>
 __global__ __launch_bounds__(256) void dp_sum_kernel(const T* __restrict__ o, const T* __restrict__ d_o,
-                                                     float* __restrict__ dsum, int64_t rows, int H) {
+                                                     float* __restrict__ dsum, int64_t rows, int H,
+                                                     const float* __restrict__ lse, float* __restrict__ lse2) {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63;
@@ -42,7 +45,10 @@ __global__ __launch_bounds__(256) void dp_sum_kernel(const T* __restrict__ o, co
   }
 #pragma unroll
   for (int off = LPR / 2; off >= 1; off >>= 1) s += __shfl_xor(s, off);
-  if (row < rows && lane % LPR == 0) dsum[row] = s;
+  if (row < rows && lane % LPR == 0) {
+    dsum[row] = s;
+    if (lse2) lse2[row] = lse[row] * 1.4426950408889634f;
+  }
 }
 
 // P[u, f, t] = exp(scale * S + bias - lse[f]); masked entries (causal: t > f) are zero.
@@ -137,6 +143,8 @@ bool fused_path(uint64_t units, uint32_t H, uint32_t F, uint32_t T, bool maybe_b
 }
 
 size_t dsum_bytes(uint64_t units, uint64_t F) { return ((size_t)units * F * sizeof(float) + 255) & ~(size_t)255; }
+// Scratch of the fused path: rowsum(dO o O), then LSE * log2(e), one float per query row each.
+size_t fused_bytes(uint64_t units, uint64_t F) { return 2 * dsum_bytes(units, F); }
 
 template <typename T>
 int run(const void* q, const void* k, const void* v, const void* bias, const void* o, const void* d_o,
@@ -149,20 +157,22 @@ int run(const void* q, const void* k, const void* v, const void* bias, const voi
   const T* Q = (const T*)q; const T* K = (const T*)k; const T* V = (const T*)v; const T* dO = (const T*)d_o;
   T* dQ = (T*)dq; T* dK = (T*)dk; T* dV = (T*)dv;
   const int64_t rows = units * F;
+  const bool fused = fused_path((uint64_t)units, (uint32_t)H, (uint32_t)F, (uint32_t)Tk, bias != nullptr);
+  float* lse2 = reinterpret_cast<float*>(ws + dsum_bytes((uint64_t)units, (uint64_t)F));  // fused path only
   if (H <= 64)
     hipLaunchKernelGGL((dp_sum_kernel<T, 8>), dim3((unsigned)xmk::ceil_div(rows, 32)), dim3(256), 0, st, (const T*)o, dO,
-                       dsum, rows, (int)H);
+                       dsum, rows, (int)H, fused ? lse : nullptr, fused ? lse2 : nullptr);
   else if (H <= 128)
     hipLaunchKernelGGL((dp_sum_kernel<T, 16>), dim3((unsigned)xmk::ceil_div(rows, 16)), dim3(256), 0, st, (const T*)o, dO,
-                       dsum, rows, (int)H);
+                       dsum, rows, (int)H, fused ? lse : nullptr, fused ? lse2 : nullptr);
   else
     hipLaunchKernelGGL((dp_sum_kernel<T, 32>), dim3((unsigned)xmk::ceil_div(rows, 8)), dim3(256), 0, st, (const T*)o, dO,
-                       dsum, rows, (int)H);
+                       dsum, rows, (int)H, fused ? lse : nullptr, fused ? lse2 : nullptr);
   // The gradients come from the fused kernels, which keep the scores on chip;
   // XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
   {
-    const fmha_bwd_fused::Args a{q, k, v, d_o, bias, lse, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
-    if (fused_path((uint64_t)units, (uint32_t)H, (uint32_t)F, (uint32_t)Tk, bias != nullptr)) {
+    const fmha_bwd_fused::Args a{q, k, v, d_o, bias, lse2, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
+    if (fused) {
       fmha_bwd_fused::launch(a, (uint64_t)units, dtype == XMK_BF16, st);
       return xmk::check_launch("fmha_bwd");
     }
@@ -212,7 +222,7 @@ extern "C" size_t xmk_fmha_bwd_workspace_bytes(uint32_t num_batches, uint32_t nu
   if (check_dims(num_batches, num_heads, head_size, num_queries, num_keys) != XMK_OK) return 0;
   const uint64_t units = (uint64_t)num_batches * num_heads;
   // The fused kernels keep the scores on chip; only the GEMM composition needs the score-sized buffers.
-  if (fused_path(units, head_size, num_queries, num_keys, true)) return dsum_bytes(units, num_queries);
+  if (fused_path(units, head_size, num_queries, num_keys, true)) return fused_bytes(units, num_queries);
   return make_plan(units, num_queries, num_keys).total;
 }
 
@@ -232,7 +242,7 @@ extern "C" int xmk_fmha_bwd(const void* query, const void* key, const void* valu
     return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_bwd: head_scale must be positive and finite");
   const uint64_t units = (uint64_t)num_batches * num_heads;
   const Plan pl = make_plan(units, num_queries, num_keys);
-  const size_t need = fused_path(units, head_size, num_queries, num_keys, bias != nullptr) ? dsum_bytes(units, num_queries)
+  const size_t need = fused_path(units, head_size, num_queries, num_keys, bias != nullptr) ? fused_bytes(units, num_queries)
                                                                                           : pl.total;
   if (workspace_bytes < need)
     return xmk::fail(XMK_INVALID_ARGUMENT, "fmha_bwd: workspace of %zu bytes, %zu needed", workspace_bytes, need);

@@ -13,7 +13,7 @@ struct Args {
   const void* v;
   const void* d_o;
   const void* bias;   // [units, F, T] additive bias or null
-  const float* lse;   // [units, F] log-sum-exp of the forward pass (natural log)
+  const float* lse;   // [units, F] log-sum-exp of the forward pass times log2(e)
   const float* dsum;  // [units, F] rowsum(dO o O)
   void* dq;
   void* dk;

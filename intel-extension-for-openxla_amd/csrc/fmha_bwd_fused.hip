@@ -81,7 +81,7 @@ struct KParams {
   const void* strm2;  // streamed operand of the dP product:    dO (owner = keys) or V
   const void* bias;   // [units, F, T] additive bias of the scores, or null
   int bias_vec;       // queries-own pass: the bias may be read 4 keys (8 bytes) at a time
-  const float* lse;   // [units, F] natural-log LSE of the forward pass
+  const float* lse;   // [units, F] LSE of the forward pass times log2(e)
   const float* dsum;  // [units, F] D = rowsum(dO o O)
   void* out1;         // scale * dS^T Q (dK)  or  scale * dS K (dQ)
   void* out2;         // P^T dO (dV), owner = keys only
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
   float own_lse2 = 0.f, own_d = 0.f;
   if constexpr (!OWNER_K) {
     if (orow < p.F) {
-      own_lse2 = lse[orow] * kLog2e;
+      own_lse2 = lse[orow];
       own_d = dsum[orow];
     }
   }
@@ -367,7 +367,7 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int i = 4 * qd + e;
-            const float lse2 = OWNER_K ? l2[e] * kLog2e : own_lse2;
+            const float lse2 = OWNER_K ? l2[e] : own_lse2;
             const float dq = OWNER_K ? dd[e] : own_d;
             float arg;
             if constexpr (BIAS) arg = __builtin_fmaf(sc[kt][i], scale2, __builtin_fmaf(bs[kt][i], kLog2e, -lse2));
