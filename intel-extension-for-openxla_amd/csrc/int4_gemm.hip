@@ -210,7 +210,8 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     u32x4 a[SPG][MT];
   };
   auto fetch = [&](int g, GroupData& d) {
-    const uint32_t so = (uint32_t)(g * N * 2);
+    // (wave-uniform; said explicitly, or the compiler wraps each of the two loads in a loop over lane values)
+    const uint32_t so = __builtin_amdgcn_readfirstlane((uint32_t)(g * N * 2));
     d.sc = load_halves<W>(r_s, voff_sz, so);
     d.zp = load_halves<W>(r_z, voff_sz, so);
 #pragma unroll
