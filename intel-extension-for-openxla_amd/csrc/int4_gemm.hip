@@ -112,7 +112,10 @@ __device__ __forceinline__ float half_at(const Words<NWORDS>& r, int c) {
 // MT   : 16-row activation tiles (1 or 2)
 // RI   : accumulator rows per lane that can be live (4, or fewer when M <= 4 so that the
 //        per-group fix-up only touches rows that exist)
-// SPG  : 32-channel k-steps per quantisation group (group = 32*SPG)
+// SPG  : 32-channel k-steps a wave handles at a time (one load batch, one fix-up)
+// SDIV : such batches per quantisation group (group = 32 * SPG * SDIV): groups of 256 channels run as two
+//        batches of 128 that read the same scale and zero point -- s (d1 - z a1) + s (d2 - z a2) -- because
+//        a batch of 256 does not fit the register file (it spilled over a hundred registers)
 // NW   : waves per block; wave w takes groups w, w+NW, ... and the partial
 //        sums meet in LDS in a fixed order (deterministic result)
 // SPREAD: 2 to 4 rows (RI = 1) or 5 to 8 rows (RI = 2): activation row r is fed to the MFMA as row
@@ -137,7 +140,7 @@ struct Int4Problem {
   float* partial;
 };
 
-template <int W, int MT, int RI, int SPG, int NW, bool SK, bool SPREAD>
+template <int W, int MT, int RI, int SPG, int NW, bool SK, bool SPREAD, int SDIV = 1>
 __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0, int mixed) {
   // mixed (two K-split products of equal width): the products alternate from one block to the next, and
   // the alternation flips between the first and the second half of the K slices, so that work-groups
@@ -167,13 +170,13 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   const int kg = lane >> 4;
   const int n0 = bx * NCOL + col16 * W;
   const bool col_ok = n0 < N;
-  const int ngroups = K / (32 * SPG);
+  const int ngroups = K / (32 * SPG);  // batches; ngroups / SDIV rows of scales and zero points
 
   // Buffer descriptors: hardware bounds checking zero-fills lanes that are out of range
   // (offset kOob), and the per-lane byte offsets below never change inside the K loop.
   const __amdgpu_buffer_rsrc_t r_w = make_rsrc(qw, (uint32_t)((size_t)(K / 8) * N * 4));
-  const __amdgpu_buffer_rsrc_t r_s = make_rsrc(scales, (uint32_t)((size_t)ngroups * N * 2));
-  const __amdgpu_buffer_rsrc_t r_z = make_rsrc(zeros, (uint32_t)((size_t)ngroups * N * 2));
+  const __amdgpu_buffer_rsrc_t r_s = make_rsrc(scales, (uint32_t)((size_t)(ngroups / SDIV) * N * 2));
+  const __amdgpu_buffer_rsrc_t r_z = make_rsrc(zeros, (uint32_t)((size_t)(ngroups / SDIV) * N * 2));
   // (the 32 rows of this launch only: the byte count must fit the descriptor's 32 bits for any M)
   const __amdgpu_buffer_rsrc_t r_a = make_rsrc(act + (size_t)m_base * K, (uint32_t)((size_t)min(M - m_base, 32) * K * 2));
   const uint32_t voff_w = col_ok ? (uint32_t)((kg * N + n0) * 4) : kOob;
@@ -211,7 +214,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   };
   auto fetch = [&](int g, GroupData& d) {
     // (wave-uniform; said explicitly, or the compiler wraps each of the two loads in a loop over lane values)
-    const uint32_t so = __builtin_amdgcn_readfirstlane((uint32_t)(g * N * 2));
+    const uint32_t so = __builtin_amdgcn_readfirstlane((uint32_t)((g / SDIV) * N * 2));
     d.sc = load_halves<W>(r_s, voff_sz, so);
     d.zp = load_halves<W>(r_z, voff_sz, so);
 #pragma unroll
@@ -395,7 +398,7 @@ struct Config {
   bool operator==(const Config& o) const { return w == o.w && nw == o.nw && ksplit == o.ksplit; }
 };
 
-template <int W, int MT, int RI, int SPG, int NW, bool SPREAD>
+template <int W, int MT, int RI, int SPG, int NW, bool SPREAD, int SDIV = 1>
 void launch(const Int4Problem& a, const Int4Problem* b, int ksplit, hipStream_t st) {
   const int blocks0 = (int)xmk::ceil_div(a.N, 16 * W);
   const int blocks = blocks0 + (b ? (int)xmk::ceil_div(b->N, 16 * W) : 0);
@@ -403,12 +406,12 @@ void launch(const Int4Problem& a, const Int4Problem* b, int ksplit, hipStream_t 
   if (ksplit > 1) {
     if constexpr (W == 4 && MT == 1) {  // the only shape the split is planned for
       const int mixed = b && blocks == 2 * blocks0 && ksplit % 4 == 0 ? 1 : 0;
-      hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true, SPREAD>), dim3(blocks, ksplit), dim3(NW * 64), 0, st, a,
+      hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, true, SPREAD, SDIV>), dim3(blocks, ksplit), dim3(NW * 64), 0, st, a,
                          second, blocks0, mixed);
       return;
     }
   }
-  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false, SPREAD>), dim3(blocks), dim3(NW * 64), 0, st, a, second,
+  hipLaunchKernelGGL((int4_gemm_kernel<W, MT, RI, SPG, NW, false, SPREAD, SDIV>), dim3(blocks), dim3(NW * 64), 0, st, a, second,
                      blocks0, 0);
 }
 
@@ -418,7 +421,7 @@ int launch_spg(int spg, const Int4Problem& a, const Int4Problem* b, int ksplit, 
     case 1: launch<W, MT, RI, 1, NW, SPREAD>(a, b, ksplit, st); break;
     case 2: launch<W, MT, RI, 2, NW, SPREAD>(a, b, ksplit, st); break;
     case 4: launch<W, MT, RI, 4, NW, SPREAD>(a, b, ksplit, st); break;
-    case 8: launch<W, MT, RI, 8, NW, SPREAD>(a, b, ksplit, st); break;
+    case 8: launch<W, MT, RI, 4, NW, SPREAD, 2>(a, b, ksplit, st); break;  // groups of 256: two batches of 128
     default: return xmk::fail(XMK_UNIMPLEMENTED, "int4_gemm: group must be 32, 64, 128 or 256");
   }
   return XMK_OK;
