@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
     // The dK launch of the larger head sizes holds both owner operands, the accumulators and the scores of
     // a whole block only with spills (30 registers): it goes through the block's two halves one after the
     // other, so that one half's scores are dead before the other's are made.
-    constexpr bool BY_HALF = DS && !PV && ((OWNER_K && HP >= 128) || HP > 128);
+    constexpr bool BY_HALF = DS && ((OWNER_K && HP >= 128) || HP > 128);
     floatx16 sc[2], dp[2];
     if constexpr (!BY_HALF) {
       scores(c1, of1, sc);
