@@ -218,6 +218,40 @@ __global__ __launch_bounds__(NT) void fmha_decode_merge_kernel(DecodeParams p) {
   }
 }
 
+// Up to 16 splits (what 64 and more units plan): no LDS and no barrier.  Every thread loads all the
+// splits' statistics (the same few cache lines for the whole work-group) and its own column of the partial
+// outputs in one go, so the kernel costs one round of loads instead of three dependent ones.
+constexpr int SMALL_SPLITS = 16;
+template <typename T>
+__global__ __launch_bounds__(NT) void fmha_decode_merge_small_kernel(DecodeParams p) {
+  const int unit = blockIdx.x, H = p.H, S = p.splits;
+  const int64_t stride = H + 2;
+  const float* wsu = p.ws + (int64_t)unit * S * stride;
+  const int h = threadIdx.x < H ? threadIdx.x : 0;
+  float ms[SMALL_SPLITS], ls[SMALL_SPLITS], os[SMALL_SPLITS];
+#pragma unroll
+  for (int s = 0; s < SMALL_SPLITS; ++s) {
+    const bool ok = s < S;
+    ms[s] = ok ? wsu[s * stride + H] : -INFINITY;
+    ls[s] = ok ? wsu[s * stride + H + 1] : 0.f;
+    os[s] = ok ? wsu[s * stride + h] : 0.f;
+  }
+  float m = ms[0];
+#pragma unroll
+  for (int s = 1; s < SMALL_SPLITS; ++s) m = fmaxf(m, ms[s]);
+  // Same order of additions as the general kernel for up to 16 splits: four interleaved partial sums.
+  float l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < SMALL_SPLITS; ++s) {
+    const float w = ms[s] > -INFINITY ? __builtin_amdgcn_exp2f(ms[s] - m) : 0.f;
+    l += ls[s] * w;
+    if (s < (S & ~3)) o[s & 3] += os[s] * w;
+    else o[0] += os[s] * w;
+  }
+  if (threadIdx.x < H)
+    reinterpret_cast<T*>(p.out)[(int64_t)unit * H + threadIdx.x] = (T)(((o[0] + o[1]) + (o[2] + o[3])) / l);
+}
+
 void plan(uint32_t units, uint32_t T, int* splits, int* chunk) {
   // About 1024 work-groups in flight (XMK_DECODE_WGS overrides the target), at least 64 and at most
   // 512 keys per chunk.
@@ -241,7 +275,10 @@ void launch(const DecodeParams& p, int units, hipStream_t st) {
   if (p.H <= 64) hipLaunchKernelGGL((fmha_decode_split_kernel<T, 8>), grid, block, 0, st, p);
   else if (p.H <= 128) hipLaunchKernelGGL((fmha_decode_split_kernel<T, 16>), grid, block, 0, st, p);
   else hipLaunchKernelGGL((fmha_decode_split_kernel<T, 32>), grid, block, 0, st, p);
-  hipLaunchKernelGGL((fmha_decode_merge_kernel<T>), dim3((unsigned)units), block, 0, st, p);
+  if (p.splits <= SMALL_SPLITS && p.H <= NT)
+    hipLaunchKernelGGL((fmha_decode_merge_small_kernel<T>), dim3((unsigned)units), block, 0, st, p);
+  else
+    hipLaunchKernelGGL((fmha_decode_merge_kernel<T>), dim3((unsigned)units), block, 0, st, p);
 }
 
 }  // namespace
