@@ -31,6 +31,17 @@ __global__ __launch_bounds__(LN_NT) void layernorm_kernel(const _Float16* __rest
   union Pack { ln_u32x4 u; _Float16 e[8]; };
   const _Float16* xr = x + (size_t)blockIdx.x * d;
   Pack v[LN_MAXV];
+  // gamma and beta do not depend on the statistics: fetched up front, their latency passes under the row's
+  // (a load cannot move up across the barrier below by itself)
+  Pack gm[LN_MAXV], bt[LN_MAXV];
+#pragma unroll
+  for (int j = 0; j < LN_MAXV; ++j) {
+    const int i = (threadIdx.x + j * LN_NT) * 8;
+    if (i < d) {
+      gm[j].u = *reinterpret_cast<const ln_u32x4*>(gamma + i);
+      bt[j].u = *reinterpret_cast<const ln_u32x4*>(beta + i);
+    }
+  }
   float s = 0.f, ss = 0.f;
 #pragma unroll
   for (int j = 0; j < LN_MAXV; ++j) {
@@ -103,12 +114,10 @@ __global__ __launch_bounds__(LN_NT) void layernorm_kernel(const _Float16* __rest
   for (int j = 0; j < LN_MAXV; ++j) {
     const int i = (threadIdx.x + j * LN_NT) * 8;
     if (i < d) {
-      Pack g, b, o;
-      g.u = *reinterpret_cast<const ln_u32x4*>(gamma + i);
-      b.u = *reinterpret_cast<const ln_u32x4*>(beta + i);
+      Pack o;
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        o.e[e] = (_Float16)(((float)v[j].e[e] - mean) * rstd * (float)g.e[e] + (float)b.e[e]);
+        o.e[e] = (_Float16)(((float)v[j].e[e] - mean) * rstd * (float)gm[j].e[e] + (float)bt[j].e[e]);
       *reinterpret_cast<ln_u32x4*>(y + (size_t)blockIdx.x * d + i) = o.u;
     }
   }
