@@ -494,14 +494,21 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
           asm volatile("" : XMK_ACC(ot[ht]));
         }
       };
-      // Elements 2k, 2k+1 of S_h: exponentials, rounding to one packed word of P_h, row-sum share.
-      auto epiece = [&](auto KC) {
+      // Elements 2k, 2k+1 of S_h: exponentials, rounding to one packed word of P_h, row-sum share.  In two
+      // halves one slot apart: a transcendental's result costs a wait state when the very next vector
+      // instruction uses it, so the rounding of piece k runs behind the exponentials of piece k + 1.
+      float e0[8], e1[8];
+      auto epiece_exp = [&](auto KC) {
         constexpr int k = decltype(KC)::value;
         float x0 = sc[2 * k], x1 = sc[2 * k + 1];
         asm volatile("" : "+v"(x0), "+v"(x1));
-        const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, p.scale2, -mref_c));
-        const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, p.scale2, -mref_c));
-        const T r0 = (T)e0, r1 = (T)e1;
+        e0[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, p.scale2, -mref_c));
+        e1[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, p.scale2, -mref_c));
+        asm volatile("" : "+v"(e0[k]), "+v"(e1[k]));
+      };
+      auto epiece_round = [&](auto KC) {
+        constexpr int k = decltype(KC)::value;
+        const T r0 = (T)e0[k], r1 = (T)e1[k];
         l_run = Elem<T>::dot2_ones(r0, r1, l_run);
         pf[k / 4][2 * (k % 4)] = r0;
         pf[k / 4][2 * (k % 4) + 1] = r1;
@@ -525,12 +532,17 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
         fetch(std::integral_constant<int, i + D>{});
         fire(I);
         static_for<8>([&](auto KC) {
-          if constexpr ((decltype(KC)::value * NSLOT) / 8 == i) epiece(KC);
+          constexpr int k = decltype(KC)::value;
+          if constexpr ((k * NSLOT) / 8 == i) {
+            epiece_exp(KC);
+            if constexpr (k > 0) epiece_round(std::integral_constant<int, (k > 0 ? k - 1 : 0)>{});
+          }
         });
         if constexpr (sco && i == R0) rpiece0();
         if constexpr (sco && i == R1) rpiece1();
         __builtin_amdgcn_sched_barrier(0);
       });
+      epiece_round(std::integral_constant<int, 7>{});
       static_for<2>([&](auto U) {
         u32x4 w = __builtin_bit_cast(u32x4, pf[decltype(U)::value]);
         asm volatile("" : "+v"(w));
