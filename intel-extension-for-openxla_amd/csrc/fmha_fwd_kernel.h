@@ -350,10 +350,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
       }
     }
     if constexpr (decltype(MASKED)::value) {
+      // Most masked steps of a wave have nothing to mask (the half tile lies below the wave's rows and inside
+      // the keys): a wave-uniform test skips those.  Otherwise both limits fold into one threshold per lane
+      // and an element costs a compare with a constant and a select.
+      if ((CAUSAL && k0 + 31 > wq0) || k0 + 32 > Tk) {
+        const int thr = min(CAUSAL ? qrow : 0x7fffffff, Tk - 1) - k0 - 4 * g;  // key offsets above it are masked
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = k0 + 8 * (i / 4) + 4 * g + (i % 4);
-        if ((CAUSAL && key > qrow) || key >= Tk) st[i] = -INFINITY;
+        for (int i = 0; i < 16; ++i)
+          if (8 * (i / 4) + (i % 4) > thr) st[i] = -INFINITY;
       }
     }
   };
@@ -433,7 +437,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   //   - waits until the loads that the NEXT step reads have landed (those sent two steps ago: the
   //     loads of this and the last step may stay in flight) and meets the other waves.
   // MASKED steps: S_{h+1} touches the causal diagonal or the end of the keys; they also check every
-  // load against the end of K / V and wait for all loads, and a wave leaves out the work past its
+  // load against the end of K / V and wait for all loads (counting the loads that the last steps still send,
+  // and waiting only for the older ones, was measured: no gain), and a wave leaves out the work past its
   // last half tile (nh).  PV / SC: whether there is a P V product (not in step 0) and an S product
   // (not in the last step) to run.
   float mref_c, alpha_c = 1.0f;  // exponent reference of S_h; factor O has to be multiplied by before P V of h
