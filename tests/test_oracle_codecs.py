@@ -73,7 +73,7 @@ def test_e4m3fn_encode(oracle):
     gn, rn = (got & 0x7F) == 0x7F, (ref & 0x7F) == 0x7F
     assert np.array_equal(gn, rn)
     assert np.array_equal(got[~gn], ref[~rn])
-    # the three probes the survey recorded for torch's cast
+    # three known values of torch's cast (0.3, 448, 1e-3)
     probe = oracle.to_f32(oracle.from_f32(np.array([0.3, 448.0, 1e-3], np.float32),
                                           oracle.F8E4M3FN), oracle.F8E4M3FN)
     assert probe.tolist() == [0.3125, 448.0, 0.001953125]
