@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Roofline benchmark of the custom-call kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also] [--no-cpu] [--ramp S]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-also] [--no-cpu] [--ramp S] [--observe S]
 
 One JSON line on stdout.  A "step" is one launch of the workload's kernel on synthetic inputs that
 are already resident in HBM.  The headline workload is benchmark configuration 2 (fused causal MHA forward,
@@ -31,6 +31,167 @@ TRAFFIC_BYTES = {
     "int4_m1": (17480 * 2.0 + 32) * 1024,
     "fp8_8192": (393600 * 2.0 + 131100) * 1024,
 }
+
+
+class Seeded:
+    """The deterministic input generator of the parity tests, restated on the GPU: a splitmix64 counter
+    hash (seed, element index) -> 64 bits; N(0,1) by Box-Muller in double on counters 2i, 2i+1;
+    U(lo,hi) and 32-bit words from counter i.  Same seed and shape give the values the tests' host
+    generator gives (up to the last bit of the device's log / cos before the cast to float)."""
+    CHUNK = 1 << 24
+
+    def __init__(self, torch):
+        self.t = torch
+        s = lambda v: torch.tensor(v - (1 << 64) if v >= (1 << 63) else v, dtype=torch.int64, device="cuda")
+        self.c1, self.c2, self.c3 = s(0x9e3779b97f4a7c15), s(0xbf58476d1ce4e5b9), s(0x94d049bb133111eb)
+        self.m, self.a = s(0xd1342543de82ef95), s(0x632be59bd9b4e019)
+
+    @staticmethod
+    def _lsr(x, k):  # logical shift right of the 64-bit pattern held in an int64
+        return (x >> k) & ((1 << (64 - k)) - 1)
+
+    def _mix(self, x):
+        x = x + self.c1
+        x = (x ^ self._lsr(x, 30)) * self.c2
+        x = (x ^ self._lsr(x, 27)) * self.c3
+        return x ^ self._lsr(x, 31)
+
+    def _draw(self, seed, ctr):
+        key = self._mix(self.t.tensor(seed, dtype=self.t.int64, device="cuda"))
+        return self._mix(key ^ (ctr * self.m + self.a))
+
+    def _unit(self, r):  # (0, 1)
+        return (self._lsr(r, 11).double() + 0.5) * (1.0 / 9007199254740992.0)
+
+    def _chunks(self, n):
+        for lo in range(0, n, self.CHUNK):
+            yield lo, self.t.arange(lo, min(n, lo + self.CHUNK), dtype=self.t.int64, device="cuda")
+
+    def normal(self, shape, seed, scale=1.0, dtype=None):
+        t = self.t
+        n = 1
+        for d in shape:
+            n *= d
+        out = t.empty((n,), dtype=dtype or t.float32, device="cuda")
+        for lo, i in self._chunks(n):
+            u1, u2 = self._unit(self._draw(seed, 2 * i)), self._unit(self._draw(seed, 2 * i + 1))
+            z = t.sqrt(-2.0 * t.log(u1)) * t.cos(6.283185307179586476925 * u2)
+            out[lo:lo + i.numel()] = (z * float(scale)).float().to(out.dtype)  # double -> float -> storage type
+        return out.view(shape)
+
+    def uniform(self, shape, seed, lo_v, hi_v, dtype=None):
+        t = self.t
+        n = 1
+        for d in shape:
+            n *= d
+        out = t.empty((n,), dtype=dtype or t.float32, device="cuda")
+        lo_f, hi_f = (t.tensor(v, dtype=t.float32).item() for v in (lo_v, hi_v))  # the bounds are floats, widened
+        for lo, i in self._chunks(n):
+            u = self._unit(self._draw(seed, i))
+            out[lo:lo + i.numel()] = (lo_f + u * (hi_f - lo_f)).float().to(out.dtype)
+        return out.view(shape)
+
+    def words(self, shape, seed):
+        t = self.t
+        n = 1
+        for d in shape:
+            n *= d
+        out = t.empty((n,), dtype=t.int32, device="cuda")
+        for lo, i in self._chunks(n):
+            out[lo:lo + i.numel()] = self._lsr(self._draw(seed, i), 32).to(t.int32)  # low 32 bits kept: wraps to signed
+        return out.view(shape)
+
+
+_GEN = None
+
+
+def gen(torch):
+    global _GEN
+    if _GEN is None:
+        _GEN = Seeded(torch)
+    return _GEN
+
+
+class ClockSampler:
+    """Core clock (per XCD) and socket power as the SMI library reports them, read by a host thread
+    while a workload runs untimed: what the device held under that load, next to the published peak
+    (which assumes 2400 MHz).  Never running during a timed region."""
+
+    def __init__(self):
+        self.smi = self.handle = None
+        self.source = "unavailable"
+        try:
+            sys.path.insert(0, "/opt/rocm/share/amd_smi")
+            import amdsmi
+            amdsmi.amdsmi_init()
+            self.handle = amdsmi.amdsmi_get_processor_handles()[0]
+            self.smi = amdsmi
+            self.source = "amdsmi gpu_metrics (current_gfxclks, current_socket_power)"
+            if not self._read():
+                self.source = "amdsmi clock_info / power_info"
+                self.metrics = False
+                if not self._read():
+                    self.smi, self.source = None, "unavailable"
+        except Exception as e:  # no SMI library, or no permission: the bench line says so
+            self.smi, self.source = None, f"unavailable ({type(e).__name__})"
+
+    metrics = True
+
+    def _read(self):
+        try:
+            if self.metrics:
+                m = self.smi.amdsmi_get_gpu_metrics_info(self.handle)
+                clks = [c for c in m.get("current_gfxclks", []) if isinstance(c, (int, float)) and 0 < c < 10000]
+                pw = m.get("current_socket_power")
+                if not clks:
+                    return None
+                return clks, (pw if isinstance(pw, (int, float)) and pw < 10000 else None)
+            c = self.smi.amdsmi_get_clock_info(self.handle, self.smi.AmdSmiClkType.GFX)["clk"]
+            pw = self.smi.amdsmi_get_power_info(self.handle).get("current_socket_power")
+            return [c], (pw if isinstance(pw, (int, float)) else None)
+        except Exception:
+            return None
+
+    def observe(self, torch, fn, seconds):
+        """Runs fn back to back for `seconds` and samples every ~10 ms; returns the summary dict."""
+        if self.smi is None or seconds <= 0:
+            return {"source": self.source}
+        import threading
+        samples, stop = [], threading.Event()
+
+        def loop():
+            while not stop.is_set():
+                r = self._read()
+                if r:
+                    samples.append(r)
+                time.sleep(0.01)
+        th = threading.Thread(target=loop, daemon=True)
+        t0 = time.perf_counter()
+        started = False
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(8):
+                fn()
+            torch.cuda.synchronize()
+            if not started and time.perf_counter() - t0 > 0.3 * seconds:  # sample the settled part only
+                th.start()
+                started = True
+        stop.set()
+        if started:
+            th.join()
+        if not samples:
+            return {"source": self.source, "samples": 0}
+        means = [sum(c) / len(c) for c, _ in samples]
+        pws = [p for _, p in samples if p is not None]
+        out = {"source": self.source, "samples": len(samples), "mean_mhz": round(sum(means) / len(means)),
+               "min_mhz": round(min(min(c) for c, _ in samples)), "max_mhz": round(max(max(c) for c, _ in samples)),
+               "xcds": len(samples[0][0])}
+        if pws:
+            out["socket_power_w_mean"] = round(sum(pws) / len(pws))
+        return out
+
+
+CLOCKS = None
+OBSERVE_SECONDS = 0.5
 
 
 def _events(torch, fn, steps, warmup, graph=False):
@@ -79,7 +240,7 @@ def _events(torch, fn, steps, warmup, graph=False):
 
 # ---------------------------------------------------------------- workloads
 def wl_fmha(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
-    q, k, v = (torch.randn((B, N, S, H), device="cuda").bfloat16() for _ in range(3))
+    q, k, v = (gen(torch).normal((B, N, S, H), 201 + i, dtype=torch.bfloat16) for i in range(3))
     out = torch.empty_like(q)
     flops = 4.0 * B * N * S * S * H * (0.5 if causal else 1.0)
     nbytes = 4.0 * B * N * S * H * 2
@@ -92,7 +253,7 @@ def wl_fmha(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
 def wl_fmha_bwd(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
     """Gradients of the headline attention shape.  Flops counted as the 5 products of the textbook
     backward (2.5x the forward's), although the kernels recompute S per pass."""
-    q, k, v, d_o = (torch.randn((B, N, S, H), device="cuda").bfloat16() for _ in range(4))
+    q, k, v, d_o = (gen(torch).normal((B, N, S, H), 201 + i, dtype=torch.bfloat16) for i in range(4))
     out = torch.empty_like(q)
     lse = torch.empty((B * N, S), dtype=torch.float32, device="cuda")
     xmk.fmha_forward(q, k, v, out, lse=lse, causal=causal)
@@ -104,9 +265,9 @@ def wl_fmha_bwd(torch, xmk, causal=True, B=8, N=32, S=2048, H=128):
 
 
 def wl_gemm(torch, xmk, m, n, k, bias=False, rhs_t=False):
-    a = (torch.randn((m, k), device="cuda") * k ** -0.5).bfloat16()
-    b = (torch.randn((n, k) if rhs_t else (k, n), device="cuda") * k ** -0.5).bfloat16()
-    bv = (torch.randn((n,), device="cuda") * k ** -0.5).bfloat16() if bias else None
+    a = gen(torch).normal((m, k), 101, k ** -0.5, dtype=torch.bfloat16)
+    b = gen(torch).normal((n, k) if rhs_t else (k, n), 102, k ** -0.5, dtype=torch.bfloat16)
+    bv = gen(torch).normal((n,), 103, k ** -0.5, dtype=torch.bfloat16) if bias else None
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     epi = xmk.EPI_BIAS if bias else xmk.EPI_DEFAULT
     return dict(name=f"gemm_bf16_{m}x{n}x{k}{'_bias' if bias else ''}{'_rhsT' if rhs_t else ''}",
@@ -116,8 +277,8 @@ def wl_gemm(torch, xmk, m, n, k, bias=False, rhs_t=False):
 
 
 def wl_fp8(torch, xmk, m, n, k, rhs_t=True):
-    a = torch.randn((m, k), device="cuda")
-    b = torch.randn((n, k) if rhs_t else (k, n), device="cuda")
+    a = gen(torch).normal((m, k), 401)
+    b = gen(torch).normal((n, k) if rhs_t else (k, n), 402)
     sa, sb = a.abs().max() / 448.0, b.abs().max() / 448.0
     qa, qb = (a / sa).to(torch.float8_e4m3fn), (b / sb).to(torch.float8_e4m3fn)
     sa, sb = sa.reshape(1).float(), sb.reshape(1).float()
@@ -131,11 +292,11 @@ def wl_fp8(torch, xmk, m, n, k, rhs_t=True):
 def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
     # Rotate through `copies` weight sets (12 x 35.7 MB > the 256 MB last-level cache) so that
     # every launch streams its weights from HBM.
-    qws = [torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 8, n), dtype=torch.int32, device="cuda")
-           for _ in range(copies)]
-    sc = [(torch.rand((k // group, n), device="cuda") * 0.019 + 0.001).half() for _ in range(copies)]
-    zp = [(torch.rand((k // group, n), device="cuda") * 15).half() for _ in range(copies)]
-    act = torch.randn((m, k), device="cuda").half()
+    G = gen(torch)
+    qws = [G.words((k // 8, n), 300 + 10 * c) for c in range(copies)]
+    sc = [G.uniform((k // group, n), 301 + 10 * c, 0.001, 0.02, dtype=torch.float16) for c in range(copies)]
+    zp = [G.uniform((k // group, n), 302 + 10 * c, 0.0, 15.0, dtype=torch.float16) for c in range(copies)]
+    act = G.normal((m, k), 299, dtype=torch.float16)
     out = torch.empty((m, n), dtype=torch.float16, device="cuda")
     state = [0]
 
@@ -148,6 +309,28 @@ def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
                 bound="hbm", dtype="f16", kernel="int4_gemm_kernel", graph=True)
 
 
+def wl_gemv_f16(torch, xmk, m=1, n=16384, k=4096, copies=4):
+    """Dense fp16 small-row GEMM, the shape class the reference's own tile table is mostly made of
+    (`1_16384_4096`, xla/service/gpu/xetla/gemm/gemm.cc:33): weight-bandwidth bound, so reported as
+    HBM GB/s.  K-split through xmk_gemm_ws with caller scratch when the planner asks for one.  The
+    launches rotate through `copies` weight sets (4 x 134 MB > the 256 MB last-level cache)."""
+    G = gen(torch)
+    a = G.normal((m, k), 601, dtype=torch.float16)
+    bs = [G.normal((k, n), 602 + c, k ** -0.5, dtype=torch.float16) for c in range(copies)]
+    out = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    need = xmk.gemm_workspace_bytes(a, bs[0], out)
+    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device="cuda") if need else None
+    state = [0]
+
+    def fn():
+        b = bs[state[0] % copies]
+        state[0] += 1
+        xmk.run_gemm(a, b, out, workspace=ws)
+    return dict(name=f"gemm_f16_m{m}_n{n}_k{k}", fn=fn, flops=2.0 * m * n * k, bytes=2.0 * (m * k + k * n + m * n),
+                bound="hbm", dtype="f16", kernel="gemm_mfma_kernel (+ splitk_reduce_kernel)", graph=True,
+                note=f"xmk_gemm_ws, {need} bytes of K-split scratch" if need else "xmk_gemm, unsplit")
+
+
 def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
     """benchmark configuration 5: GPT-J-6B-shaped decode step, int4 group-128 weights, fp16 KV cache filled to
     `cache_len`, one new token per sequence.  The whole step (about 8 launches per block) is replayed
@@ -155,11 +338,17 @@ def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
     d, heads, hd, dff, vocab, g = 4096, 16, 256, 16384, 50400, 128
     cap = cache_len + 1
 
+    G, seed = gen(torch), [500]
+
+    def nxt():
+        seed[0] += 1
+        return seed[0]
+
     def lin(k, n, bias):
-        qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 8, n), dtype=torch.int32, device="cuda")
-        sc = (torch.rand((k // g, n), device="cuda") * 0.019 + 0.001).half()
-        zp = (torch.rand((k // g, n), device="cuda") * 15).half()
-        b = (torch.randn((n,), device="cuda") * 0.02).half() if bias else None
+        qw = G.words((k // 8, n), nxt())
+        sc = G.uniform((k // g, n), nxt(), 0.001, 0.02, dtype=torch.float16)
+        zp = G.uniform((k // g, n), nxt(), 0.0, 15.0, dtype=torch.float16)
+        b = G.normal((n,), nxt(), 0.02, dtype=torch.float16) if bias else None
         return qw, sc, zp, b
 
     layers = []
@@ -167,12 +356,12 @@ def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
         layers.append(dict(ln_gamma=torch.ones((d,), device="cuda").half(), ln_beta=torch.zeros((d,), device="cuda").half(),
                            qkv=lin(d, 3 * d, False), out_proj=lin(d, d, False), fc_in=lin(d, dff, True),
                            fc_out=lin(dff, d, True),
-                           k_cache=torch.randn((batch, heads, cap, hd), device="cuda").half(),
-                           v_cache=torch.randn((batch, heads, cap, hd), device="cuda").half()))
+                           k_cache=G.normal((batch, heads, cap, hd), nxt(), dtype=torch.float16),
+                           v_cache=G.normal((batch, heads, cap, hd), nxt(), dtype=torch.float16)))
     cfg = xmk.GptjConfig(n_layer, heads, hd, 64, d, dff, vocab, g, batch, cap, 1e-5)
     dec = xmk.GptjDecoder(cfg, layers, torch.ones((d,), device="cuda").half(), torch.zeros((d,), device="cuda").half(),
                           lin(d, vocab, True))
-    hidden = torch.randn((batch, d), device="cuda").half()
+    hidden = G.normal((batch, d), nxt(), dtype=torch.float16)
     logits = torch.empty((batch, vocab), dtype=torch.float16, device="cuda")
     wbytes = n_layer * ((4 * d * d + 2 * d * dff) / 2 + (4 * d * d + 2 * d * dff) / g * 4) \
         + d * vocab / 2 + d * vocab / g * 4
@@ -185,8 +374,8 @@ def wl_gptj_decode(torch, xmk, n_layer=28, batch=4, cache_len=2047):
 def wl_lib_gemm(torch, xmk, m=8192, n=8192, k=8192):
     """torch.matmul (hipBLASLt / rocBLAS behind it) on the 8192^3 shape: what the vendor library reaches on
     the same device in the same run, to read the GEMM kernel's fraction of the published peak against."""
-    a = (torch.randn((m, k), device="cuda") * k ** -0.5).bfloat16()
-    b = (torch.randn((k, n), device="cuda") * k ** -0.5).bfloat16()
+    a = gen(torch).normal((m, k), 101, k ** -0.5, dtype=torch.bfloat16)
+    b = gen(torch).normal((k, n), 102, k ** -0.5, dtype=torch.bfloat16)
     out = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     return dict(name=f"library_torch_matmul_bf16_{m}x{n}x{k}", fn=lambda: torch.matmul(a, b, out=out), flops=2.0 * m * n * k,
                 bytes=2.0 * (m * k + k * n + m * n), bound="mfma", dtype="bf16", kernel="vendor library GEMM (not this library)")
@@ -210,6 +399,8 @@ WORKLOADS = {
     "gemm_8192_rhsT": lambda t, x: wl_gemm(t, x, 8192, 8192, 8192, rhs_t=True),
     "gemm_c1": lambda t, x: wl_gemm(t, x, 512, 4096, 4096, bias=True),
     "lib_gemm_8192": lambda t, x: wl_lib_gemm(t, x),
+    "gemv_f16_m1": lambda t, x: wl_gemv_f16(t, x, 1),
+    "gemv_f16_m4_vocab": lambda t, x: wl_gemv_f16(t, x, 4, 50400, 4096, copies=2),
     "int4_m1": lambda t, x: wl_int4(t, x, 1),
     "int4_m8": lambda t, x: wl_int4(t, x, 8),
     "int4_m32": lambda t, x: wl_int4(t, x, 32),
@@ -217,7 +408,7 @@ WORKLOADS = {
     "fp8_8192_kn": lambda t, x: wl_fp8(t, x, 8192, 8192, 8192, rhs_t=False),
     "gptj_decode": lambda t, x: wl_gptj_decode(t, x),
 }
-ALSO = ["fmha", "fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "lib_gemm_8192", "gemm_c1", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "fp8_8192_kn", "gptj_decode"]
+ALSO = ["fmha", "fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "lib_gemm_8192", "gemm_c1", "gemv_f16_m1", "gemv_f16_m4_vocab", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "fp8_8192_kn", "gptj_decode"]
 
 
 def measure(torch, xmk, key, steps, warmup):
@@ -232,6 +423,9 @@ def measure(torch, xmk, key, steps, warmup):
     roof = {"bound": w["bound"], "achieved": round(achieved, 2), "peak": peak, "unit": unit,
             "frac": round(achieved / peak, 4), "traffic": TRAFFIC_BYTES.get(key), "kernel": w["kernel"],
             "kernel_ms": round(ms, 5), "algorithmic_flops": w["flops"], "algorithmic_bytes": w["bytes"]}
+    if CLOCKS is not None:
+        # after the timed region: the same launches back to back while a host thread reads the SMI clocks
+        roof["clock_mhz_observed"] = CLOCKS.observe(torch, w["fn"], OBSERVE_SECONDS)
     return w, ms, wall_ms, roof
 
 
@@ -360,6 +554,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--ramp", type=float, default=RAMP_SECONDS,
                     help="seconds of untimed launches before the warmup steps (0 for profiler runs)")
+    ap.add_argument("--observe", type=float, default=0.5,
+                    help="seconds each workload runs untimed, after its timed steps, while the SMI clocks are sampled "
+                         "(0: no sampling, for profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1",
@@ -372,6 +569,9 @@ def main():
     xmk.lib()  # fails loudly if libxmk.so is missing: there is no fallback path
     torch.cuda.set_device(0)
 
+    if args.observe > 0:
+        globals()["CLOCKS"] = ClockSampler()
+        globals()["OBSERVE_SECONDS"] = args.observe
     w, ms, wall_ms, roof = measure(torch, xmk, args.workload, args.steps, args.warmup)
     line = {
         "metric": "TFLOP/s & %MFMA peak (GEMM/MHA); int4 GEMV HBM GB/s & %peak; 1 GPU",
@@ -396,7 +596,10 @@ def main():
     try:
         props = torch.cuda.get_device_properties(0)
         line["device"] = {"name": props.name, "cus": props.multi_processor_count,
-                          "clock_mhz": getattr(props, "clock_rate", 0) // 1000}
+                          "clock_mhz_assumed_by_peak": 2400,
+                          "clock_mhz_observed": roof.get("clock_mhz_observed", {"source": "not sampled (--observe 0)"}),
+                          "note": "the published peaks assume 2400 MHz; each workload's roofline entry carries the clock the "
+                                  "SMI library reported while that workload ran"}
     except Exception:  # device query is informational only
         pass
     print(json.dumps(line), flush=True)

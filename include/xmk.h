@@ -203,8 +203,13 @@ int xmk_fmha_decode(const void* query, const void* key, const void* value, void*
  * whose xmk_fmha_decode_workspace_bytes() exceeds xmk_fmha_decode_static_max_bytes() are rejected with
  * XMK_INVALID_ARGUMENT.  All calls on one GPU share that GPU's array: calls that overlap in time on
  * one GPU (different streams, or threads) race; calls ordered on one stream are safe.  The device
- * the stream belongs to must be the calling thread's current device. */
+ * the stream belongs to must be the calling thread's current device.
+ * The first call on a device looks up the array's device address (hipGetSymbolAddress), which makes
+ * the runtime load the library's code object there if it has not yet: not something to do under
+ * stream capture.  xmk_fmha_decode_static_init() does that lookup for the calling thread's current
+ * device and nothing else; call it (or make one ordinary call) on each device before capturing. */
 size_t xmk_fmha_decode_static_max_bytes(void);
+int xmk_fmha_decode_static_init(void);
 int xmk_fmha_decode_static(const void* query, const void* key, const void* value, void* out,
                            int32_t dtype, uint32_t num_batches, uint32_t num_heads,
                            uint32_t head_size, uint32_t num_keys, int64_t kv_head_stride,
@@ -251,6 +256,14 @@ int xmk_int4_dequant(const void* qweight, const void* scales, const void* zeros,
 int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                  void* out, int64_t m, int64_t n, int64_t k, int32_t rhs_transpose,
                  void* stream);
+
+/* The same product with the rest of the "__cublas$lt$matmul$f8" operand list applied on the device:
+ * out = bf16(d_scale * (a_scale * b_scale * A B + bias)).  d_scale (device fp32 scalar) and bias
+ * (bf16 [N]) may each be NULL.  The reference's handlers use every operand they are handed
+ * (xla/service/gpu/sycl_custom_call.cc:168-205); this is the entry point the f8 handler calls. */
+int xmk_fp8_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                    const float* d_scale, const void* bias, void* out, int64_t m, int64_t n,
+                    int64_t k, int32_t rhs_transpose, void* stream);
 
 /* ------------------------------------------------------------------------
  * GPT-J-shaped decode step on int4 weights: one new token per sequence through

@@ -39,7 +39,9 @@ XLA_FFI_Error* xmk_ffi_cublas_lt_matmul(XLA_FFI_CallFrame* call_frame);
  * K [.., T, H], V [.., T, H] [, bias [B,N,F,T]]) -> results (out [.., F, H], scratch
  * [, activation f32 [B,N,F]]).  Attributes (all optional): fmha_scale f64|f32 (default 1),
  * dropout_rate f64|f32 (must be 0, :57-61), is_causal_mask pred|i32 (default 0).  A scale above
- * 1 is replaced by 1/sqrt(H) as the reference does (:129). */
+ * 1 is replaced by 1/sqrt(H) as the reference does (:129).  Rank 3 (one batch, the batch dimension
+ * left out) is accepted beside the rank 4 the reference's runner CHECKs for (:114-116), in the
+ * forward and the backward handlers alike; every operand's element count must match the shape. */
 XLA_FFI_Error* xmk_ffi_fmha_softmax(XLA_FFI_CallFrame* call_frame);
 XLA_FFI_Error* xmk_ffi_fmha_scale_bias_softmax(XLA_FFI_CallFrame* call_frame);
 
@@ -59,9 +61,13 @@ XLA_FFI_Error* xmk_ffi_fmha_scale_bias_softmax_backward(XLA_FFI_CallFrame* call_
 XLA_FFI_Error* xmk_ffi_int4_gemm(XLA_FFI_CallFrame* call_frame);
 
 /* "__cublas$lt$matmul$f8" (not in the reference snapshot; XLA's operand convention): operands
- * (a f8e4m3fn, b f8e4m3fn, a_scale f32[], b_scale f32[] [, further scales, ignored]) -> results
- * (out bf16, ...).  Attributes as for "__cublas$lt$matmul"; lhs row-major, beta 0, alpha 1,
- * epilogue DEFAULT. */
+ * (a f8e4m3fn, b f8e4m3fn, a_scale f32[], b_scale f32[] [, c_scale f32[], d_scale f32[]] [, bias
+ * bf16 [N]]) -> results (out bf16, ...), out = bf16(d_scale * (a_scale * b_scale * A B + bias)).
+ * The bias is there exactly when the epilogue is BIAS.  c_scale multiplies the matrix addend, which
+ * this target does not take (beta must be 0), so its value has no effect.  Every other operand
+ * count, a matrix addend (beta != 0) and every other epilogue are rejected with UNIMPLEMENTED or
+ * INVALID_ARGUMENT: no operand is dropped silently.  Attributes as for "__cublas$lt$matmul"; lhs
+ * and output row-major, alpha 1, batch 1. */
 XLA_FFI_Error* xmk_ffi_cublas_lt_matmul_f8(XLA_FFI_CallFrame* call_frame);
 
 typedef struct xmk_ffi_target {

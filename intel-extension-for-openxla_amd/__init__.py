@@ -235,6 +235,11 @@ def fmha_decode_static_max_bytes():
     return lib().xmk_fmha_decode_static_max_bytes()
 
 
+def fmha_decode_static_init():
+    """Looks up the built-in scratch array on the current device (to be done before stream capture)."""
+    _check(lib().xmk_fmha_decode_static_init())
+
+
 # ----------------------------------------------------------------------- int4
 def int4_gemm(act, qweight, scales, zeros, out, *, group=128, bias=None, stream=None):
     m, k = act.shape
@@ -270,12 +275,18 @@ def int4_dequant(qweight, scales, zeros, w_out, *, group=128, stream=None):
 
 
 # ------------------------------------------------------------------------ fp8
-def fp8_gemm(a, b, a_scale, b_scale, out, *, rhs_transpose=False, stream=None):
+def fp8_gemm(a, b, a_scale, b_scale, out, *, rhs_transpose=False, d_scale=None, bias=None, stream=None):
+    """out = bf16(d_scale * (a_scale * b_scale * a b + bias)); d_scale / bias given: xmk_fp8_gemm_ex."""
     m, k = a.shape
     n = b.shape[0] if rhs_transpose else b.shape[1]
-    _check(lib().xmk_fp8_gemm(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(out),
-                              ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
-                              ctypes.c_int32(int(rhs_transpose)), _stream(stream)))
+    if d_scale is None and bias is None:
+        _check(lib().xmk_fp8_gemm(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(out),
+                                  ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
+                                  ctypes.c_int32(int(rhs_transpose)), _stream(stream)))
+    else:
+        _check(lib().xmk_fp8_gemm_ex(_ptr(a), _ptr(b), _ptr(a_scale), _ptr(b_scale), _ptr(d_scale), _ptr(bias),
+                                     _ptr(out), ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
+                                     ctypes.c_int32(int(rhs_transpose)), _stream(stream)))
     return out
 
 

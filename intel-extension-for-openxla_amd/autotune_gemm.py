@@ -8,8 +8,8 @@ csrc/gemm_policy_table.h with the shapes where the heuristic's choice is not the
 slices (xmk_gemm_ws with scratch; XMK_GEMM_SPLITK forces the slices) and merges the winners into the table.
 
 The counterpart of the reference's tuned table (xetla/gemm/gemm.cc:31-285) and of its
-GemmAlgorithmPicker measurement loop (gemm_impl_picker.cc:124-185).  One worker process per
-policy (XMK_GEMM_POLICY is read once per process); the parent never touches the GPU.
+GemmAlgorithmPicker measurement loop (gemm_impl_picker.cc:124-185).  The measurements run in worker
+processes (XMK_GEMM_POLICY / XMK_GEMM_SPLITK force a choice); the parent never touches the GPU.
 Rebuild the library afterwards (python build.py) for the table to take effect.
 """
 import argparse
@@ -36,7 +36,11 @@ DEFAULT_SHAPES = [(m, n, k) for m in MS for (n, k) in NK] + [(8192, 8192, 8192)]
 # projections (4096 x 4096, 4096 -> 16384, 16384 -> 4096, the stacked q/k/v 4096 -> 12288).
 SMALL_NK = [(4096, 16384), (16384, 4096), (4096, 4096), (12288, 4096)]
 SMALL_MS = [1, 4, 8, 16, 32]
-SMALL_SHAPES = [(m, n, k) for m in SMALL_MS for (n, k) in SMALL_NK]
+# The vocabulary projections that fill the reference's table for m = 1, 4 (gemm.cc:77-80, 92-93, 112-113);
+# 50400 = 787.5 x 64 is ragged in every tile width.
+VOCAB_NK = [(50400, 4096), (50272, 4096), (32000, 4096), (65024, 4096)]
+VOCAB_MS = [1, 4, 32]
+SMALL_SHAPES = [(m, n, k) for m in SMALL_MS for (n, k) in SMALL_NK] + [(m, n, k) for m in VOCAB_MS for (n, k) in VOCAB_NK]
 SPLITS = [1, 2, 4, 8, 16]
 
 
@@ -56,45 +60,56 @@ def heuristic(m, n, k):
 
 
 def worker_small(shapes):
-    """Times xmk_gemm_ws (scratch for up to 16 slices) from a HIP graph of 20 launches per replay."""
+    """Times xmk_gemm_ws (scratch for up to 16 slices) from a HIP graph of 20 launches per replay, for the
+    library's own choice and for every tile policy x number of K slices (XMK_GEMM_POLICY / XMK_GEMM_SPLITK
+    are read at every call, so one process walks them all)."""
     sys.path.insert(0, os.path.dirname(HERE))
     import torch
     xmk = importlib.import_module(os.path.basename(HERE))
-    out = {}
+    cands = [None] + [(pol, ks) for pol in range(len(POLICIES)) for ks in SPLITS]
+    out = {("default" if c is None else f"{c[0]}x{c[1]}"): {} for c in cands}
     for (m, n, k) in shapes:
         a = (torch.randn((m, k), device="cuda") * k ** -0.5).bfloat16()
-        bs = [(torch.randn((k, n), device="cuda") * k ** -0.5).bfloat16() for _ in range(4)]  # rotate past the cache
+        copies = max(2, min(4, int(6e8 // (2 * n * k)) + 1))  # rotate past the 256 MB cache
+        bs = [(torch.randn((k, n), device="cuda") * k ** -0.5).bfloat16() for _ in range(copies)]
         c = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
         ws = torch.empty((16 * m * n,), dtype=torch.float32, device="cuda")
-        st = torch.cuda.Stream()
-        with torch.cuda.stream(st):
-            for b in bs:
-                xmk.run_gemm(a, b, c, workspace=ws)
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=st):
-                for i in range(20):
-                    xmk.run_gemm(a, bs[i % 4], c, workspace=ws)
-        torch.cuda.synchronize()
-        g.replay()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        best = 1e30
-        for _ in range(5):
-            s.record()
-            g.replay()
-            e.record()
+        for cand in cands:
+            for var in ("XMK_GEMM_POLICY", "XMK_GEMM_SPLITK"):
+                os.environ.pop(var, None)
+            if cand is not None:
+                os.environ["XMK_GEMM_POLICY"], os.environ["XMK_GEMM_SPLITK"] = str(cand[0]), str(cand[1])
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                for b in bs:
+                    xmk.run_gemm(a, b, c, workspace=ws)
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=st):
+                    for i in range(20):
+                        xmk.run_gemm(a, bs[i % copies], c, workspace=ws)
             torch.cuda.synchronize()
-            best = min(best, s.elapsed_time(e) / 20)
-        out[f"{m},{n},{k}"] = best
+            g.replay()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            best = 1e30
+            for _ in range(5):
+                s.record()
+                g.replay()
+                e.record()
+                torch.cuda.synchronize()
+                best = min(best, s.elapsed_time(e) / 20)
+            out["default" if cand is None else f"{cand[0]}x{cand[1]}"][f"{m},{n},{k}"] = best
+            del g
+        print(f"shape {m},{n},{k} measured", file=sys.stderr, flush=True)
     print("RESULT " + json.dumps(out), flush=True)
 
 
 def run_worker(shapes, env_extra, flag):
     env = dict(os.environ, **env_extra)
     cmd = [sys.executable, os.path.abspath(__file__), flag, "--shapes"] + [f"{m},{n},{k}" for m, n, k in shapes]
-    r = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=900)
+    r = subprocess.run(cmd, env=env, stdout=subprocess.PIPE, text=True, timeout=1100)
     line = [l for l in r.stdout.splitlines() if l.startswith("RESULT ")]
     if r.returncode != 0 or not line:
-        sys.exit(f"worker {env_extra} failed:\n{r.stdout[-2000:]}\n{r.stderr[-2000:]}")
+        sys.exit(f"worker {env_extra} failed:\n{r.stdout[-2000:]}")
     return json.loads(line[0][7:])
 
 
@@ -124,19 +139,16 @@ def write_table(rows):
 
 
 def tune_small(shapes, args):
-    base = run_worker(shapes, {}, "--worker-small")
-    print("default choice measured", flush=True)
-    cand = {}
-    for pol in range(len(POLICIES)):
-        for ks in SPLITS:
-            cand[(pol, ks)] = run_worker(shapes, {"XMK_GEMM_POLICY": str(pol), "XMK_GEMM_SPLITK": str(ks)}, "--worker-small")
-            print(f"policy {pol} x {ks} slices measured", flush=True)
+    res = run_worker(shapes, {}, "--worker-small")
+    base = res.pop("default")
+    cand = {tuple(int(x) for x in key.split("x")): v for key, v in res.items()}
     rows = load_table()
     for (m, n, k) in shapes:
         key = f"{m},{n},{k}"
         best = min(cand, key=lambda c: cand[c][key])
         t0, t1 = base[key] * 1e3, cand[best][key] * 1e3
-        print(f"{key:>18}: default {t0:7.2f} us  best {t1:7.2f} us  = {POLICIES[best[0]]} x {best[1]} slices")
+        gbs = 2.0 * (m * k + k * n + m * n) / t0 / 1e3
+        print(f"{key:>18}: default {t0:7.2f} us ({gbs:5.0f} GB/s)  best {t1:7.2f} us  = {POLICIES[best[0]]} x {best[1]} slices")
         rows.pop((m, n, k), None)
         if t1 < t0 * (1.0 - args.margin):
             rows[(m, n, k)] = (best[0], best[1], f"{t0:.1f} -> {t1:.1f} us")

@@ -270,7 +270,8 @@ XLA_FFI_Error* fmha_common(XLA_FFI_CallFrame* f, bool with_bias) {
   const int64_t N = q->dims[rank - 3], F = q->dims[rank - 2], H = q->dims[rank - 1];
   const int64_t T = k->dims[rank - 2];
   if (k->dims[rank - 1] != H || v->dims[rank - 1] != H || v->dims[rank - 2] != T || k->dims[rank - 3] != N ||
-      v->dims[rank - 3] != N || elements(out) != B * N * F * H || (bias && elements(bias) != B * N * F * T) ||
+      v->dims[rank - 3] != N || elements(q) != B * N * F * H || elements(k) != B * N * T * H ||
+      elements(v) != B * N * T * H || elements(out) != B * N * F * H || (bias && elements(bias) != B * N * F * T) ||
       (act && elements(act) != B * N * F))
     fr.fail(XMK_INVALID_ARGUMENT, "fmha: operand shapes do not agree");
   if (q->dtype != k->dtype || q->dtype != v->dtype || q->dtype != out->dtype || (bias && bias->dtype != q->dtype))
@@ -318,7 +319,8 @@ XLA_FFI_Error* fmha_bwd_common(XLA_FFI_CallFrame* f, bool with_bias) {
   const int64_t N = q->dims[rank - 3], F = q->dims[rank - 2], H = q->dims[rank - 1];
   const int64_t T = k->dims[rank - 2];
   if (k->dims[rank - 1] != H || v->dims[rank - 1] != H || v->dims[rank - 2] != T || k->dims[rank - 3] != N ||
-      v->dims[rank - 3] != N || elements(d_out) != B * N * F * H || elements(fwd_out) != B * N * F * H ||
+      v->dims[rank - 3] != N || elements(k) != B * N * T * H || elements(v) != B * N * T * H ||
+      elements(d_out) != B * N * F * H || elements(fwd_out) != B * N * F * H ||
       elements(act) != B * N * F || elements(dq) != B * N * F * H || elements(dk) != B * N * T * H ||
       elements(dv) != B * N * T * H || (bias && elements(bias) != B * N * F * T))
     fr.fail(XMK_INVALID_ARGUMENT, "fmha backward: operand shapes do not agree");
@@ -405,17 +407,31 @@ extern "C" XLA_FFI_Error* xmk_ffi_cublas_lt_matmul_f8(XLA_FFI_CallFrame* f) {
   const XLA_FFI_Buffer* b_scale = fr.arg(3);
   const XLA_FFI_Buffer* out = fr.ret(0);
   if (fr.code != XMK_OK) return finish(fr, XMK_OK);
+  const int epilogue = fr.has("epilogue") ? as_xmk_epilogue(fr.i64("epilogue")) : XMK_EPI_DEFAULT;
+  if (epilogue != XMK_EPI_DEFAULT && epilogue != XMK_EPI_BIAS)
+    fr.fail(XMK_UNIMPLEMENTED, "matmul$f8: epilogue must be DEFAULT or BIAS");
+  if (fr.f64("beta") != 0.0 || fr.f64("alpha") != 1.0 || fr.i64("batch_size") != 1)
+    fr.fail(XMK_UNIMPLEMENTED, "matmul$f8: needs alpha 1, beta 0 (no matrix addend), batch 1");
+  // Operands after b_scale: [c_scale, d_scale] [, bias].  Like the reference's handlers
+  // (sycl_custom_call.cc:168-205) every operand handed over is either used or refused.
+  const bool with_bias = epilogue == XMK_EPI_BIAS;
+  const int64_t rest = f->args.size - 4 - (with_bias ? 1 : 0);
+  if (fr.code == XMK_OK && rest != 0 && rest != 2)
+    fr.fail(XMK_INVALID_ARGUMENT, "matmul$f8: " + std::to_string(f->args.size) + " operands do not fit (a, b, a_scale, "
+            "b_scale [, c_scale, d_scale] [, bias]) with epilogue " + (with_bias ? "BIAS" : "DEFAULT"));
+  if (fr.code != XMK_OK) return finish(fr, XMK_OK);
+  const XLA_FFI_Buffer* c_scale = rest == 2 ? fr.arg(4) : nullptr;
+  const XLA_FFI_Buffer* d_scale = rest == 2 ? fr.arg(5) : nullptr;
+  const XLA_FFI_Buffer* bias = with_bias ? fr.arg(4 + rest) : nullptr;
+  if (fr.code != XMK_OK) return finish(fr, XMK_OK);
   if (a->dtype != XLA_FFI_DataType_F8E4M3FN || b->dtype != XLA_FFI_DataType_F8E4M3FN)
     fr.fail(XMK_UNIMPLEMENTED, "matmul$f8: operands must be f8e4m3fn");
   if (out->dtype != XLA_FFI_DataType_BF16) fr.fail(XMK_UNIMPLEMENTED, "matmul$f8: output must be bf16");
-  if (a_scale->dtype != XLA_FFI_DataType_F32 || b_scale->dtype != XLA_FFI_DataType_F32 || elements(a_scale) != 1 ||
-      elements(b_scale) != 1)
-    fr.fail(XMK_INVALID_ARGUMENT, "matmul$f8: a_scale and b_scale must be f32 scalars");
+  for (const XLA_FFI_Buffer* s : {a_scale, b_scale, c_scale, d_scale})
+    if (s && (s->dtype != XLA_FFI_DataType_F32 || elements(s) != 1))
+      fr.fail(XMK_INVALID_ARGUMENT, "matmul$f8: a_scale, b_scale, c_scale and d_scale must be f32 scalars");
   if (fr.i64("lhs_order") != 0 || fr.i64("output_order") != 0)
     fr.fail(XMK_UNIMPLEMENTED, "matmul$f8: lhs and output must be row-major");
-  if (fr.f64("beta") != 0.0 || fr.f64("alpha") != 1.0 || fr.i64("batch_size") != 1 ||
-      (fr.has("epilogue") && fr.i64("epilogue") != 0))
-    fr.fail(XMK_UNIMPLEMENTED, "matmul$f8: needs alpha 1, beta 0, batch 1, epilogue DEFAULT");
   const int64_t M = fr.i64("lhs_num_rows"), K = fr.i64("lhs_num_cols"), N = fr.i64("rhs_num_cols");
   const int rhs_t = fr.i64("rhs_order") == 1;  // column-major [k,n] is stored as [n,k]
   if (fr.code == XMK_OK && (fr.i64("rhs_num_rows") != K || elements(a) != M * K || elements(b) != K * N ||
@@ -423,10 +439,14 @@ extern "C" XLA_FFI_Error* xmk_ffi_cublas_lt_matmul_f8(XLA_FFI_CallFrame* f) {
                             fr.i64("rhs_leading_dim_stride") != (rhs_t ? K : N) ||
                             fr.i64("output_leading_dim_stride") != N))
     fr.fail(XMK_INVALID_ARGUMENT, "matmul$f8: shapes do not agree or operands are not packed");
+  if (bias && (bias->dtype != XLA_FFI_DataType_BF16 || elements(bias) != N))
+    fr.fail(XMK_INVALID_ARGUMENT, "matmul$f8: bias must be bf16 [N]");
   void* stream = fr.stream();
   if (fr.code != XMK_OK) return finish(fr, XMK_OK);
-  return finish(fr, xmk_fp8_gemm(a->data, b->data, static_cast<const float*>(a_scale->data),
-                                 static_cast<const float*>(b_scale->data), out->data, M, N, K, rhs_t, stream));
+  return finish(fr, xmk_fp8_gemm_ex(a->data, b->data, static_cast<const float*>(a_scale->data),
+                                    static_cast<const float*>(b_scale->data),
+                                    d_scale ? static_cast<const float*>(d_scale->data) : nullptr,
+                                    bias ? bias->data : nullptr, out->data, M, N, K, rhs_t, stream));
 }
 
 extern "C" const xmk_ffi_target* xmk_ffi_targets(int32_t* count) {

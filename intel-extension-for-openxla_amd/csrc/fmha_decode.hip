@@ -239,7 +239,10 @@ __global__ __launch_bounds__(NT) void fmha_decode_merge_small_kernel(DecodeParam
   float m = ms[0];
 #pragma unroll
   for (int s = 1; s < SMALL_SPLITS; ++s) m = fmaxf(m, ms[s]);
-  // Same order of additions as the general kernel for up to 16 splits: four interleaved partial sums.
+  // The partial outputs are added as four interleaved partial sums, like the general kernel's; l is
+  // added split by split (the general kernel reduces per-thread shares across the work-group) and the
+  // result is divided by l (there: multiplied by 1 / l), so the two kernels may differ in the last
+  // bit of the 16-bit result.
   float l = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < SMALL_SPLITS; ++s) {
@@ -252,14 +255,19 @@ __global__ __launch_bounds__(NT) void fmha_decode_merge_small_kernel(DecodeParam
     reinterpret_cast<T*>(p.out)[(int64_t)unit * H + threadIdx.x] = (T)(((o[0] + o[1]) + (o[2] + o[3])) / l);
 }
 
-void plan(uint32_t units, uint32_t T, int* splits, int* chunk) {
-  // About 1024 work-groups in flight (XMK_DECODE_WGS overrides the target), at least 64 and at most
-  // 512 keys per chunk.
+// Work-groups the split kernel aims to have in flight (XMK_DECODE_WGS overrides the 1024).
+uint32_t plan_target() {
   static const int target = [] {
     const char* e = getenv("XMK_DECODE_WGS");
     const int v = e ? atoi(e) : 0;
     return v >= 64 && v <= 65536 ? v : 1024;
   }();
+  return (uint32_t)target;
+}
+
+void plan(uint32_t units, uint32_t T, int* splits, int* chunk) {
+  // About plan_target() work-groups in flight, at least 64 and at most 512 keys per chunk.
+  const uint32_t target = plan_target();
   int s = (int)((target + units - 1) / units);
   int c = (int)((T + s - 1) / s);
   if (c < 64) c = 64;
@@ -275,7 +283,10 @@ void launch(const DecodeParams& p, int units, hipStream_t st) {
   if (p.H <= 64) hipLaunchKernelGGL((fmha_decode_split_kernel<T, 8>), grid, block, 0, st, p);
   else if (p.H <= 128) hipLaunchKernelGGL((fmha_decode_split_kernel<T, 16>), grid, block, 0, st, p);
   else hipLaunchKernelGGL((fmha_decode_split_kernel<T, 32>), grid, block, 0, st, p);
-  if (p.splits <= SMALL_SPLITS && p.H <= NT)
+  // XMK_DECODE_MERGE_GENERAL (read at every call, so that a test can compare the two merge kernels on one
+  // shape in one process) sends every shape to the general kernel.
+  const char* general = getenv("XMK_DECODE_MERGE_GENERAL");
+  if (p.splits <= SMALL_SPLITS && p.H <= NT && !(general && *general && *general != '0'))
     hipLaunchKernelGGL((fmha_decode_merge_small_kernel<T>), dim3((unsigned)units), block, 0, st, p);
   else
     hipLaunchKernelGGL((fmha_decode_merge_kernel<T>), dim3((unsigned)units), block, 0, st, p);
@@ -296,14 +307,13 @@ extern "C" size_t xmk_fmha_decode_cache_workspace_bytes(uint32_t num_batches, ui
                                                         uint32_t head_size, uint32_t cache_capacity) {
   // The split count is not monotonic in the number of keys (the chunk is rounded to 32 and clamped
   // to 64..512 keys), so a cache is sized for the largest count any fill level 1..capacity plans.
+  // With s = plan()'s split target per unit: up to 64 s keys the chunk is 64 and the count
+  // ceil(t / 64) <= s; up to 512 s keys the chunk is at least t / s, so the count stays <= s (and
+  // t = 64 s reaches s); beyond, the chunk is 512 and the count ceil(t / 512) grows with t.
   const uint32_t units = num_batches * num_heads;
   if (units == 0 || cache_capacity == 0) return 0;
-  int most = 0;
-  for (uint32_t t = 1; t <= cache_capacity; ++t) {
-    int splits, chunk;
-    plan(units, t, &splits, &chunk);
-    most = std::max(most, splits);
-  }
+  const uint64_t s = (plan_target() + units - 1) / units, cap = cache_capacity;
+  const uint64_t most = cap <= 512 * s ? std::min((cap + 63) / 64, s) : (cap + 511) / 512;
   return (size_t)units * most * (head_size + 2) * sizeof(float);
 }
 
@@ -390,6 +400,11 @@ int static_scratch(float** out) {
 }  // namespace
 
 extern "C" size_t xmk_fmha_decode_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int xmk_fmha_decode_static_init(void) {
+  float* ws = nullptr;
+  return static_scratch(&ws);
+}
 
 extern "C" int xmk_fmha_decode_static(const void* query, const void* key, const void* value, void* out,
                                       int32_t dtype, uint32_t num_batches, uint32_t num_heads,

@@ -1,4 +1,5 @@
-// FP8 (OCP e4m3fn) GEMM: out = bf16(a_scale * b_scale * A B), fp32 accumulation.
+// FP8 (OCP e4m3fn) GEMM: out = bf16(d_scale * (a_scale * b_scale * A B + bias)), fp32 accumulation;
+// d_scale and bias are optional.
 //
 // MFMA kernel: A [M,K] row-major and B stored [N,K] (both reduction-contiguous, the
 // layout XLA's "__cublas$lt$matmul$f8" rewrite produces).  256x256 output tile per
@@ -33,9 +34,25 @@ struct Fp8Params {
   const uint8_t* b;
   const float* a_scale;
   const float* b_scale;
+  const float* d_scale;  // optional: multiplies the result after the bias
+  const __bf16* bias;    // optional: [N], added to a_scale * b_scale * A B
   __bf16* out;
   int M, N, K;
   int tiles_m, tiles_n;
+};
+
+// out element = bf16(d_scale * (a_scale * b_scale * acc + bias[n])); `scale` = a_scale * b_scale.
+struct Fp8Epilogue {
+  float scale, post;
+  const __bf16* bias;
+  __device__ __forceinline__ explicit Fp8Epilogue(const Fp8Params& p)
+      : scale(p.a_scale[0] * p.b_scale[0]), post(p.d_scale ? p.d_scale[0] : 1.0f), bias(p.bias) {}
+  __device__ __forceinline__ bool plain() const { return !bias && post == 1.0f; }
+  __device__ __forceinline__ __bf16 operator()(float acc, int n) const {
+    float v = acc * scale;
+    if (bias) v += (float)bias[n];
+    return (__bf16)(v * post);
+  }
 };
 
 // Per-lane LDS byte offsets of an operand's fragments: lane l of the 32-row slab t gets row
@@ -220,9 +237,11 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
   __builtin_amdgcn_s_waitcnt(gemm_impl::vmcnt_imm(0));  // drain the zero-fill loads before LDS is released
 
   // acc[i][j][e] is out[m][n], m = m0 + wm WTM + 32 i + lane%32, n = n0 + wn WTN + 32 j + 8 (e/4) + 4 (lane/32) + e%4.
-  const float scale = p.a_scale[0] * p.b_scale[0];
+  const Fp8Epilogue epi(p);
+  const float scale = epi.scale;
   static_assert(NSTAGE * STAGE >= BM * BN * 2, "the output tile is staged in the operand stages");
-  if (m0 + BM <= p.M && n0 + BN <= p.N && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(p.out) % 16 == 0) {
+  // A bias or an output scale (both rare with a bf16 result) take the direct stores below.
+  if (epi.plain() && m0 + BM <= p.M && n0 + BN <= p.N && p.N % 8 == 0 && reinterpret_cast<uintptr_t>(p.out) % 16 == 0) {
     // Tile fully inside (uniform over the work-group): round, lay out row-major in LDS and copy out
     // in whole row segments.
     gemm_impl::GemmParams q{};
@@ -246,10 +265,10 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
         const int n = n0 + wn * WTN + j * 32 + q * 8 + (lane >> 5) * 4;
         if (m < p.M && n < p.N) {  // N % 4 == 0: the four columns are all in range
           union { __bf16 e[4]; u32x2 w; } o;
-          o.e[0] = (__bf16)(t[4 * q + 0] * scale);
-          o.e[1] = (__bf16)(t[4 * q + 1] * scale);
-          o.e[2] = (__bf16)(t[4 * q + 2] * scale);
-          o.e[3] = (__bf16)(t[4 * q + 3] * scale);
+          o.e[0] = epi(t[4 * q + 0], n);
+          o.e[1] = epi(t[4 * q + 1], n + 1);
+          o.e[2] = epi(t[4 * q + 2], n + 2);
+          o.e[3] = epi(t[4 * q + 3], n + 3);
           *reinterpret_cast<u32x2*>(p.out + (int64_t)m * p.N + n) = o.w;
         }
       }
@@ -339,12 +358,13 @@ __global__ __launch_bounds__(256) void fp8_gemm_gather_kernel(Fp8Params p) {
   }
 
   // acc[i][j][e] is out[m][n], m = m0 + 32 TW wm + 32 i + lane % 32, n = n0 + 32 TW wn + 32 j + 8 (e/4) + 4 (lane/32) + e%4.
+  const Fp8Epilogue epi(p);
   gemm_impl::GemmParams q{};
   q.out = p.out;
   q.M = p.M;
   q.N = p.N;
   q.ldc = p.N;
-  q.alpha = p.a_scale[0] * p.b_scale[0];
+  q.alpha = epi.scale;
   q.act = gemm_impl::ACT_NONE;
 #pragma unroll
   for (int i = 0; i < TW; ++i) {
@@ -353,10 +373,18 @@ __global__ __launch_bounds__(256) void fp8_gemm_gather_kernel(Fp8Params p) {
     for (int j = 0; j < TW; ++j) {
       const floatx16 t = acc[i][j];
       const int nb = n0 + wn * 32 * TW + j * 32 + g * 4;
-      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[0], t[1], t[2], t[3]}, m, nb, 0);
-      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[4], t[5], t[6], t[7]}, m, nb + 8, 0);
-      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[8], t[9], t[10], t[11]}, m, nb + 16, 0);
-      gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[12], t[13], t[14], t[15]}, m, nb + 24, 0);
+      if (epi.plain()) {
+        gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[0], t[1], t[2], t[3]}, m, nb, 0);
+        gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[4], t[5], t[6], t[7]}, m, nb + 8, 0);
+        gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[8], t[9], t[10], t[11]}, m, nb + 16, 0);
+        gemm_impl::store_quad<__bf16, false>(q, gemm_impl::floatx4{t[12], t[13], t[14], t[15]}, m, nb + 24, 0);
+      } else if (m < p.M) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int n = nb + 8 * (e / 4) + e % 4;
+          if (n < p.N) p.out[(int64_t)m * p.N + n] = epi(t[e], n);
+        }
+      }
     }
   }
 }
@@ -421,13 +449,13 @@ __global__ __launch_bounds__(256) void fp8_gemm_generic_kernel(Fp8Params p, int 
     }
     __syncthreads();
   }
-  const float scale = p.a_scale[0] * p.b_scale[0];
+  const Fp8Epilogue epi(p);
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
-      if (m < p.M && n < p.N) p.out[(int64_t)m * p.N + n] = (__bf16)(acc[i][j] * scale);
+      if (m < p.M && n < p.N) p.out[(int64_t)m * p.N + n] = epi(acc[i][j], n);
     }
 }
 
@@ -436,12 +464,19 @@ __global__ __launch_bounds__(256) void fp8_gemm_generic_kernel(Fp8Params p, int 
 extern "C" int xmk_fp8_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                             void* out, int64_t m, int64_t n, int64_t k, int32_t rhs_transpose,
                             void* stream) {
+  return xmk_fp8_gemm_ex(a, b, a_scale, b_scale, nullptr, nullptr, out, m, n, k, rhs_transpose, stream);
+}
+
+extern "C" int xmk_fp8_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                               const float* d_scale, const void* bias, void* out, int64_t m, int64_t n, int64_t k,
+                               int32_t rhs_transpose, void* stream) {
   if (!a || !b || !a_scale || !b_scale || !out) return xmk::fail(XMK_INVALID_ARGUMENT, "fp8_gemm: null pointer");
   if (m <= 0 || n <= 0 || k <= 0) return xmk::fail(XMK_INVALID_ARGUMENT, "fp8_gemm: empty dimension");
   if (m > (1 << 30) || n > (1 << 30) || k > (1 << 30))
     return xmk::fail(XMK_INVALID_ARGUMENT, "fp8_gemm: dimension too large");
   Fp8Params p;
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b; p.a_scale = a_scale; p.b_scale = b_scale;
+  p.d_scale = d_scale; p.bias = (const __bf16*)bias;
   p.out = (__bf16*)out; p.M = (int)m; p.N = (int)n; p.K = (int)k;
   hipStream_t st = (hipStream_t)stream;
   // The direct-to-LDS kernel: A rows and the stored rows of B start on 16-byte boundaries and hold whole

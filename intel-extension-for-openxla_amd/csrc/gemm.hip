@@ -214,11 +214,9 @@ int plan_splitk(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k, int* po
   if (d->batch_size != 1 || n % 4 != 0) return 1;
   if (d->dtype_in != XMK_BF16 && d->dtype_in != XMK_F16) return 1;
   auto divides = [&](int ks) { return ks >= 1 && ks <= 16 && k % (ks * 8) == 0; };
-  // XMK_GEMM_SPLITK=<slices> overrides the choice (read once; the autotuner's handle).
-  static const int forced = [] {
-    const char* e = getenv("XMK_GEMM_SPLITK");
-    return e ? atoi(e) : 0;
-  }();
+  // XMK_GEMM_SPLITK=<slices> overrides the choice (read at every call; the autotuner's handle).
+  const char* forced_env = getenv("XMK_GEMM_SPLITK");
+  const int forced = forced_env ? atoi(forced_env) : 0;
   if (forced >= 1) return divides(forced) ? forced : 1;
   if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit >= 1 && divides(t->ksplit)) {
     if (t->ksplit > 1) *policy = t->policy;

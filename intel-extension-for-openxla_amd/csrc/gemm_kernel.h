@@ -672,12 +672,12 @@ inline const TunedShape* tuned_shape(int64_t m, int64_t n, int64_t k) {
   return nullptr;
 }
 inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1) {
-  static const int forced = [] {
-    const char* e = getenv("XMK_GEMM_POLICY");
-    const int v = e ? atoi(e) : -1;
-    return (e && v >= 0 && v < kNumPolicies) ? v : -1;
-  }();
-  if (forced >= 0) return forced;
+  // read at every call (a getenv costs far less than a launch), so that the autotuner can walk the
+  // policies inside one process
+  if (const char* e = getenv("XMK_GEMM_POLICY")) {
+    const int v = atoi(e);
+    if (*e && v >= 0 && v < kNumPolicies) return v;
+  }
   if (batch == 1)
     if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit <= 1) return t->policy;
   // Heuristic: the policy with the best estimated throughput = (what the tile sustains when the

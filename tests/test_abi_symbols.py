@@ -79,6 +79,15 @@ def test_decode_cache_workspace_covers_every_fill_level(lib):
                     for t in list(range(1, cap + 1, step)) + [cap])
         assert worst <= have, (units, cap, worst, have)
         assert have <= 4 * lib.xmk_fmha_decode_workspace_bytes(u32(1), u32(units), u32(256), u32(cap)) + 64 * 258 * 4
+    # the closed form is exactly the maximum over all fill levels (scanned in full here), and it does not
+    # walk the fill levels: the largest capacity a uint32 holds returns at once
+    for units, cap in ((64, 2050), (64, 1000), (64, 5000), (64, 9000), (8, 4097), (300, 777), (1, 3000),
+                       (1024, 700), (2000, 520), (3, 33), (1, 1)):
+        have = lib.xmk_fmha_decode_cache_workspace_bytes(u32(1), u32(units), u32(256), u32(cap))
+        worst = max(lib.xmk_fmha_decode_workspace_bytes(u32(1), u32(units), u32(256), u32(t)) for t in range(1, cap + 1))
+        assert have == worst, (units, cap, worst, have)
+    big = lib.xmk_fmha_decode_cache_workspace_bytes(u32(1), u32(64), u32(256), u32(0xFFFFFFFF))
+    assert big == 64 * ((0xFFFFFFFF + 511) // 512) * 258 * 4
 
 
 def test_shapes_beyond_32_bit_offsets_are_rejected_before_any_launch(lib):

@@ -29,6 +29,30 @@ def test_fmha_decode(xmk, oracle, name, B, N, T, H, cap):
     assert g <= 1e-2 and e <= 1e-2, (g, e)
 
 
+def test_merge_kernels_agree(xmk, oracle):
+    """Shapes with up to 16 key splits take the merge kernel that needs no LDS; XMK_DECODE_MERGE_GENERAL
+    sends the same shape through the general one.  Same partial results, other order of additions for the
+    row sum and a division where the other multiplies by the reciprocal: at most the last bit of the
+    16-bit result may differ (2^-10 relative for fp16)."""
+    import os
+    B, N, T, H = 4, 16, 2048, 256
+    q = torch.randn((B, N, 1, H), device="cuda").half()
+    kc = torch.randn((B, N, T, H), device="cuda").half()
+    vc = torch.randn((B, N, T, H), device="cuda").half()
+    ws = torch.empty((xmk.fmha_decode_workspace_bytes(B, N, H, T),), dtype=torch.uint8, device="cuda")
+    small, general = torch.empty_like(q), torch.empty_like(q)
+    xmk.fmha_decode(q, kc, vc, small, ws)
+    torch.cuda.synchronize()
+    os.environ["XMK_DECODE_MERGE_GENERAL"] = "1"
+    try:
+        xmk.fmha_decode(q, kc, vc, general, ws)
+        torch.cuda.synchronize()
+    finally:
+        del os.environ["XMK_DECODE_MERGE_GENERAL"]
+    d = (small.float() - general.float()).abs()
+    assert (d <= general.float().abs() * 2.0 ** -10 + 1e-7).all(), d.max().item()
+
+
 def _device_model(xmk, cfg, layers, lnf, lm_head, batch, cap):
     def lin(t):
         qw, s, z, b = t

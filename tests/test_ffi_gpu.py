@@ -247,6 +247,33 @@ def test_f8_matmul_handler(ffi, oracle):
     assert g <= 5e-2 and e <= 5e-2, (g, e)
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_f8_matmul_handler_applies_every_operand(ffi, oracle, with_bias):
+    """(a, b, a_scale, b_scale, c_scale, d_scale [, bias]): out = bf16(d_scale * (a_scale b_scale A B + bias)).
+    d_scale = 0.5 and a bias of the products' magnitude: dropping either operand misses the 5e-2 bound by far.
+    Shapes cover the direct-to-LDS kernel (k % 16 == 0, n % 4 == 0) and the gathering one (k = 200)."""
+    for (m, n, k) in ((320, 264, 208), (130, 76, 200)):
+        a, sa = oracle.fp8_quantize(oracle.normal((m, k), 52))
+        b, sb = oracle.fp8_quantize(oracle.normal((n, k), 53))  # column-major [k,n]
+        bias = oracle.from_f32(oracle.normal((n,), 54, 10.0), oracle.BF16)
+        _, prod = oracle.fp8_gemm(a, b, sa, sb, rhs_t=True)
+        ref = np.float32(0.5) * (prod + (oracle.to_f32(bias, oracle.BF16)[None, :] if with_bias else np.float32(0)))
+        da, db = to_dev(a, "f8"), to_dev(b, "f8")
+        dsa, dsb = torch.tensor(float(sa), device="cuda"), torch.tensor(float(sb), device="cuda")
+        dsc, dsd = torch.tensor(3.0, device="cuda"), torch.tensor(0.5, device="cuda")  # c_scale has no addend to scale
+        dbias = to_dev(bias, "bf16")
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        host = _host()
+        ops = [_buf(da, F.F8E4M3FN), _buf(db, F.F8E4M3FN), _buf(dsa, F.F32), _buf(dsb, F.F32), _buf(dsc, F.F32),
+               _buf(dsd, F.F32)] + ([_buf(dbias, F.BF16)] if with_bias else [])
+        f = host.frame(ops, [_buf(out, F.BF16)],
+                       F.gemm_attrs(m, n, k, F.F8E4M3FN, F.BF16, rhs_col_major=True, epilogue=1 if with_bias else 0))
+        _ok(host, ffi.xmk_ffi_cublas_lt_matmul_f8(C.byref(f)))
+        g, e = oracle.rel_err(out.float().cpu().numpy(), ref)
+        print(f"[parity] f8 handler {m}x{n}x{k} bias={with_bias}: g={g:.2e} e={e:.2e}")
+        assert g <= 5e-2 and e <= 5e-2, (m, n, k, g, e)
+
+
 def test_gemm_handler_takes_scratch_for_a_k_split(ffi, oracle):
     """A small-M product with a long reduction: with DeviceMemory_Allocate / Free in the API table the
     handler asks for exactly xmk_gemm_workspace_bytes of scratch, runs the K-split path and hands the

@@ -138,3 +138,23 @@ def test_int4_and_f8_decoding_errors(lib):
     attrs = F.gemm_attrs(64, 64, 128, F.F8E4M3FN, F.BF16, rhs_col_major=True)
     assert lib.xmk_ffi_cublas_lt_matmul_f8(C.byref(host.frame([a, b, s, s], [(F.F16, 0x4000, [64, 64])], attrs))) is not None
     assert "bf16" in host.errors[-1][1]
+    # every operand is used or refused: a fifth operand alone fits neither (.., c_scale, d_scale) nor a bias
+    # (the epilogue is DEFAULT); a bias operand needs epilogue BIAS and the other way round; GELU is not taken
+    attrs = F.gemm_attrs(64, 64, 128, F.F8E4M3FN, F.BF16, rhs_col_major=True)
+    assert lib.xmk_ffi_cublas_lt_matmul_f8(C.byref(host.frame([a, b, s, s, s], [o], attrs))) is not None
+    assert host.errors[-1][0] == 3 and "operands do not fit" in host.errors[-1][1]
+    bias = (F.BF16, 0x5000, [64])
+    assert lib.xmk_ffi_cublas_lt_matmul_f8(C.byref(host.frame([a, b, s, s, s, s, bias], [o], attrs))) is not None
+    assert host.errors[-1][0] == 3 and "operands do not fit" in host.errors[-1][1]
+    attrs = F.gemm_attrs(64, 64, 128, F.F8E4M3FN, F.BF16, rhs_col_major=True, epilogue=1)
+    assert lib.xmk_ffi_cublas_lt_matmul_f8(C.byref(host.frame([a, b, s, s, s, s], [o], attrs))) is not None
+    assert host.errors[-1][0] == 3 and "operands do not fit" in host.errors[-1][1]
+    assert lib.xmk_ffi_cublas_lt_matmul_f8(
+        C.byref(host.frame([a, b, s, s, s, s, (F.F16, 0x5000, [64])], [o], attrs))) is not None
+    assert "bias must be bf16" in host.errors[-1][1]
+    assert lib.xmk_ffi_cublas_lt_matmul_f8(
+        C.byref(host.frame([a, b, s, s, (F.F32, 0x6000, [2]), s, bias], [o], attrs))) is not None
+    assert "f32 scalars" in host.errors[-1][1]
+    attrs = F.gemm_attrs(64, 64, 128, F.F8E4M3FN, F.BF16, rhs_col_major=True, epilogue=4)
+    assert lib.xmk_ffi_cublas_lt_matmul_f8(C.byref(host.frame([a, b, s, s], [o], attrs))) is not None
+    assert host.errors[-1][0] == 12 and "epilogue" in host.errors[-1][1]

@@ -1,11 +1,14 @@
 """GPU parity: fused multi-head-attention forward through the C ABI (xmk_fmha_fwd) against the
-oracle's closed form.  Tolerance 1e-2 (bf16/fp16) on (a) the error relative to the tensor's scale and
-(b) the error relative to sum_t p_t |v_t|, the scale of the terms each output is the sum of; plus the
-reference test's own absolute bound (test/jax_ut.patch:997: atol 3e-2 bf16, 1e-2 fp16).  The
-elementwise figure with eps = rms(ref) is held to 2e-2: P is rounded to the 16-bit type before P V
-(as the reference does, fmha_forward.h:378-384), and on the first causal rows, whose few O(1) terms
-are larger than the rms of the whole unit's output, that rounding alone reaches 1.3e-2 of rms(ref)
-in bf16 (measured on every kernel version; fp16 stays below 2e-3)."""
+oracle's closed form.  Tolerance 1e-2 (bf16/fp16) on (a) the error relative to the tensor's scale,
+(b) the error relative to sum_t p_t |v_t|, the scale of the terms each output is the sum of, and
+(c) the elementwise figure with eps = rms(ref); plus the reference test's own absolute bound
+(test/jax_ut.patch:997: atol 3e-2 bf16, 1e-2 fp16).  One class of cases holds (c) to 2e-2 instead:
+bf16 with a causal mask or an additive bias.  P is rounded to the 16-bit type before P V (as the
+reference does, fmha_forward.h:378-384); a mask's first rows and a bias of N(0,1) in score units
+give rows whose softmax rests on a few keys, so that the output is a few O(1) terms, larger than the
+rms of the whole unit's output, and the rounding of their weights alone reaches 1.0e-2 (bias) to
+1.3e-2 (first causal rows) of rms(ref) in bf16 (measured on every kernel version; fp16 stays below
+2e-3 and is held to 1e-2 like bf16 without mask and bias)."""
 import numpy as np
 import pytest
 import torch
@@ -36,27 +39,33 @@ def _run(xmk, oracle, name, B, N, F, T, H, *, causal=False, use_bias=False, lse=
     got = out.float().cpu().numpy().reshape(B * N, F, H)
     assert np.isfinite(got).all()
     units = list(range(B * N)) if units is None else units
+    e_bound = 2e-2 if (name == "bf16" and (causal or use_bias)) else 1e-2
     for u in units:
+        # f_stride: one stride for every unit, or a stride per unit (sampled rows 0, s, 2 s, ...)
+        fs = f_stride[u] if isinstance(f_stride, dict) else f_stride
         _, ref, ref_lse = oracle.fmha_fwd(q, k, v, dt, scale, bias=bias, causal=causal, want_lse=True,
-                                          first_unit=u, num_units=1, f_stride=f_stride)
-        ref = ref.reshape(B * N, F, H)[u, ::f_stride]
+                                          first_unit=u, num_units=1, f_stride=fs)
+        ref = ref.reshape(B * N, F, H)[u, ::fs]
         _, ref_abs, _ = oracle.fmha_fwd(q, k, v & 0x7FFF, dt, scale, bias=bias, causal=causal,
-                                        first_unit=u, num_units=1, f_stride=f_stride)
-        ref_abs = ref_abs.reshape(B * N, F, H)[u, ::f_stride]
-        g, e = oracle.rel_err(got[u, ::f_stride], ref,
+                                        first_unit=u, num_units=1, f_stride=fs)
+        ref_abs = ref_abs.reshape(B * N, F, H)[u, ::fs]
+        g, e = oracle.rel_err(got[u, ::fs], ref,
                               label=f"fmha_fwd {name} [{B},{N},{F}x{T},{H}] causal={causal} bias={use_bias} unit {u}")
-        c = oracle.cond_err(got[u, ::f_stride], ref, ref_abs)
-        assert g <= 1e-2 and c <= 1e-2 and e <= 2e-2, (u, g, c, e)
-        assert np.abs(got[u, ::f_stride] - ref).max() <= (3e-2 if name == "bf16" else 1e-2)
+        c = oracle.cond_err(got[u, ::fs], ref, ref_abs)
+        assert g <= 1e-2 and c <= 1e-2 and e <= e_bound, (u, g, c, e)
+        assert np.abs(got[u, ::fs] - ref).max() <= (3e-2 if name == "bf16" else 1e-2)
         if lse:
-            gl = lse_t.cpu().numpy()[u, ::f_stride]
-            assert np.allclose(gl, ref_lse[u, ::f_stride], rtol=1e-3, atol=1e-3)
+            gl = lse_t.cpu().numpy()[u, ::fs]
+            assert np.allclose(gl, ref_lse[u, ::fs], rtol=1e-3, atol=1e-3)
     return out
 
 
 def test_config2_causal_bf16(xmk, oracle):
-    """benchmark configuration 2: bf16 [8,32,2048,128], causal, scale 1/sqrt(128); three units, every 8th row."""
-    _run(xmk, oracle, "bf16", 8, 32, 2048, 2048, 128, causal=True, units=[0, 101, 255], f_stride=8)
+    """benchmark configuration 2: bf16 [8,32,2048,128], causal, scale 1/sqrt(128); three units, every 7th, 9th
+    and 11th row (strides coprime to the 32 rows of a wave, so the samples walk through every lane of the
+    row tiles and every position against the key tiles)."""
+    _run(xmk, oracle, "bf16", 8, 32, 2048, 2048, 128, causal=True, units=[0, 101, 255],
+         f_stride={0: 7, 101: 9, 255: 11})
 
 
 @pytest.mark.parametrize("H", [64, 128, 256])
@@ -65,7 +74,8 @@ def test_many_key_tiles(xmk, oracle, H, causal, use_bias):
     """32 key tiles, so that the unmasked steady-state steps of the pipeline run; the bias (in score units,
     N(0,1)) makes the running reference max move in later tiles too, which exercises the deferred
     rescale of O and of the row sum."""
-    _run(xmk, oracle, "bf16", 1, 2, 2048, 2048, H, causal=causal, use_bias=use_bias, lse=True, seed=31, f_stride=4)
+    _run(xmk, oracle, "bf16", 1, 2, 2048, 2048, H, causal=causal, use_bias=use_bias, lse=True, seed=31,
+         f_stride={0: 3, 1: 5})
 
 
 def test_config2_full_size_properties(xmk, oracle):
@@ -100,7 +110,7 @@ def test_reference_mha_shapes(xmk, oracle, name, shape):
     are checked on two units and a stride of query rows so the oracle finishes in seconds."""
     b, F, T, n, h = shape
     work = F * T
-    f_stride = 1 if work <= (1 << 20) else (16 if work <= (1 << 24) else 128)
+    f_stride = 1 if work <= (1 << 20) else (13 if work <= (1 << 24) else 127)  # coprime to the 32-row tiles
     units = [0, b * n - 1] if work > (1 << 18) else None
     _run(xmk, oracle, name, b, n, F, T, h, units=units, f_stride=f_stride, seed=F + T)
 
