@@ -590,6 +590,10 @@ def main():
             w2, ms2, _, roof2 = measure(torch, xmk, key, max(10, args.steps // 2), max(3, args.warmup // 2))
             also[w2["name"]] = roof2
         line["also"] = also
+    if CLOCKS is not None and not args.no_also:
+        # The headline ran first, from an idle device, and the SMI figures lag by about a second: read its
+        # clocks again now that the device has been busy throughout.
+        roof["clock_mhz_observed"] = CLOCKS.observe(torch, w["fn"], 2 * OBSERVE_SECONDS)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(torch)
         line["cpu_baseline"]["also"]["oracle_fmha_fwd_causal"] = cpu_baseline_oracle()

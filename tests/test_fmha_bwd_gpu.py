@@ -41,7 +41,8 @@ def _run(xmk, oracle, name, B, N, F, T, H, causal, use_bias, seed=0, tol_elem=No
     torch.cuda.synchronize()
     errs = {}
     for nm, got, ref in (("dq", gq, dq), ("dk", gk, dk), ("dv", gv, dv)):
-        ge, ee = oracle.rel_err(got.float().cpu().numpy(), ref.astype(np.float32))
+        ge, ee = oracle.rel_err(got.float().cpu().numpy(), ref.astype(np.float32),
+                                label=f"fmha_bwd {nm} {name} [{B},{N},{F}x{T},{H}] causal={causal} bias={use_bias}")
         errs[nm] = (ge, ee)
         assert ge <= TOL and ee <= (tol_elem or TOL_ELEM[name]), (nm, ge, ee)
     return errs

@@ -57,10 +57,10 @@ def test_int4_gemm_gptj_mlp_shape(xmk, oracle, m):
     (7, 4096, 4096, 128, True),
     (36, 256, 72, 32, True),        # 32 rows + 4 in a second launch
     (40, 512, 264, 128, False),     # 32 rows + 8
-    # 9 to 32 rows with groups of at most 128: activations staged through LDS, weights four groups ahead
+    # 9 to 32 rows (one or two 16-row tiles per wave), group sizes 32 to 128
     (12, 1024, 1024, 32, True),     # one row tile, group 32
     (9, 512, 200, 64, False),       # ragged N
-    (25, 16384, 264, 128, True),    # 16 groups per wave: four trips round the register ring
+    (25, 16384, 264, 128, True),    # 16 groups per wave
     (32, 8192, 1024, 64, False),
     (20, 256, 72, 128, False),      # fewer groups than waves
     (31, 640, 136, 128, True),      # 5 groups: waves with one group and waves with none
