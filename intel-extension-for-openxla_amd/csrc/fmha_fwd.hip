@@ -13,7 +13,8 @@ template <typename T>
 void launch_t(const FmhaParams& p, int32_t dtype, uint64_t units, uint32_t F, bool causal, int bias, hipStream_t st) {
   // Head-size classes of the reference's policy choice (fmha_forward.h:622-646).  Four waves of 32
   // query rows, two work-groups per CU: a second 32-row tile per wave (one wave per SIMD) was
-  // measured slower (741 against 796 TFLOP/s on [8,32,2048,128]), eight waves per work-group equal.
+  // measured slower (741 against 796 TFLOP/s on [8,32,2048,128]), eight waves per work-group (half the
+  // K / V loads per row) equal, then and again on the current step (1020 against 1032).
   if (p.H <= 64) launch_cfg<T, 64, 4, 2>(p, units, F, causal, bias, st);
   else if (p.H <= 128) launch_cfg<T, 128, 4, 2>(p, units, F, causal, bias, st);
   else launch_h256(p, dtype, units, F, causal, bias, st);

@@ -362,27 +362,44 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
     }
   };
 
-  // Row max of a half tile and the move of the running reference max, without a branch: the
-  // reference m_run only moves when some row's max exceeds it by more than 2^8 (wave-uniform
-  // test), so that P stays below 256 and O needs a rescale in few steps.  Returns the exponent
-  // reference; `alpha` is the factor O still has to be multiplied by (1 when nothing moved) and
-  // `moved` says whether it differs from 1 for some row; the caller rescales l_run and, later, O.
-  // mx: the maximum of the lane's 16 scores of the half tile.
-  auto row_max_tail = [&](float mx, float& alpha, bool& moved) -> float {
-    {
-      // the other 16 keys of this row are held by lane l ^ 32
-      const uint32_t b = __builtin_bit_cast(uint32_t, mx);
-      const auto sw = __builtin_amdgcn_permlane32_swap(b, b, false, false);
-      mx = fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
-    }
-    const float mx2 = mx * p.scale2;
-    moved = __any(mx2 > m_run + 8.0f);
-    const float m_new = moved ? fmaxf(m_run, mx2) : m_run;
-    alpha = moved ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;  // first step: exp2(-inf) = 0
+  // The running reference max m_run only moves when some row's max exceeds it by more than 2^8, so
+  // that P stays below 256 and O needs a rescale in few steps.  The test is wave-uniform and the
+  // common case (nothing moves) costs an exchange with lane l ^ 32 (which holds the row's other 16
+  // keys of the half tile), a max and a compare against thr_run = (m_run + 8) / scale2, the
+  // threshold in score units; the move itself sits behind a branch.  mx: the maximum of the lane's
+  // 16 scores of the half tile.
+  float thr_run = -INFINITY;
+  const float inv_scale2 = 1.0f / p.scale2;
+  auto row_max_exceeds = [&](float& mx) -> bool {
+    // v_permlane32_swap exchanges the upper 32 lanes of its first operand with the lower 32 of its second:
+    // started from two copies of mx, the first ends as the lower half's values in both halves and the
+    // second as the upper half's.  Written out because BOTH results are needed and this compiler's
+    // __builtin_amdgcn_permlane32_swap hands back the first one twice (the max of the two then folds
+    // away and the row max would cover the lower lanes' 16 keys only).  The s_nop covers the two wait
+    // states the instruction needs after a vector write of its operands, which the hazard recogniser
+    // cannot insert inside an asm statement.
+    float other = mx;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(mx), "+v"(other));
+    mx = __builtin_elementwise_maximum(mx, other);
+    return __any(mx > thr_run);
+  };
+  // The move: returns the new exponent reference; `alpha` is the factor l and O still have to be
+  // multiplied by.
+  auto move_reference = [&](float mx, float& alpha) -> float {
+    const float m_new = fmaxf(m_run, mx * p.scale2);
+    alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // first step: exp2(-inf) = 0
     m_run = m_new;
+    thr_run = (m_new + 8.0f) * inv_scale2;
     // A row that has seen no visible key keeps m_run = -inf; use 0 as its reference so that
     // its masked (-inf) scores give exp2(-inf) = 0 and not NaN.
     return m_new == -INFINITY ? 0.0f : m_new;
+  };
+  // Maximum of an accumulator's 16 elements (v_maximum3_f32: no canonicalising copies of the inputs).
+  auto max16 = [](const floatx16& x) -> float {
+    float mx = __builtin_elementwise_maximum(x[0], x[1]);
+#pragma unroll
+    for (int i = 2; i < 16; i += 2) mx = __builtin_elementwise_maximum(__builtin_elementwise_maximum(mx, x[i]), x[i + 1]);
+    return mx;
   };
 
   // O^T += V^T P^T for the 16 keys of group ug (0, 1) of the half tile in a V stage.
@@ -458,7 +475,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
     if (!masked || h + 2 < nhalf) issue_half(std::integral_constant<bool, !masked>{}, V, h + 2, vfree, &voff, 1);
     if constexpr ((HS & 1) == 1 && sco) take_bias((h + 1) / 2);
     if (!masked || h - 1 < nh) {
-      float alpha_n = 1.0f, mref_n = 0.0f;
+      float alpha_n = 1.0f, mref_n = mref_c;
       bool moved_n = false;
       // The step is written as a sequence of slots, one per matrix instruction, each closed by a
       // scheduling fence: slot i sends the LDS fragment reads of matrix instruction i + D, issues matrix
@@ -522,14 +539,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
       float mx = 0.0f;
       auto rpiece0 = [&]() {
         bias_and_mask(MASKED, sn, h + 1, (HS & 1) ? b0 : b1);
-        mx = fmaxf(sn[0], sn[1]);
-#pragma unroll
-        for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, sn[i]), sn[i + 1]);  // v_max3_f32
+        mx = max16(sn);
         asm volatile("" : "+v"(mx));
       };
       auto rpiece1 = [&]() {
-        mref_n = row_max_tail(mx, alpha_n, moved_n);
-        asm volatile("" : "+v"(mref_n), "+v"(alpha_n));
+        moved_n = row_max_exceeds(mx);
+        asm volatile("" : "+v"(mx));
       };
       static_for<D>(fetch);
       static_for<NSLOT>([&](auto I) {
@@ -553,8 +568,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
         asm volatile("" : "+v"(w));
         pf[decltype(U)::value] = __builtin_bit_cast(V8, w);
       });
-      // l_run now holds every term up to P_h under the reference of S_h; move it to the new reference
-      l_run *= alpha_n;
+      // The rare move of the reference (wave-uniform).  l_run holds every term up to P_h under the
+      // reference of S_h: it moves to the new reference here, O a step later.
+      if (moved_n) {
+        mref_n = move_reference(mx, alpha_n);
+        l_run *= alpha_n;
+      }
       // The rare rescale of O, after the P V product of half tile h-1 and before that of half tile h.
       if (moved_c) {
 #pragma unroll
@@ -589,12 +608,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   scores(kst0, sa);
   bias_and_mask(true_type{}, sa, 0, b0);
   {
-    float a0;
-    bool mv0;
-    float mx = fmaxf(sa[0], sa[1]);
-#pragma unroll
-    for (int i = 2; i < 16; i += 2) mx = fmaxf(fmaxf(mx, sa[i]), sa[i + 1]);
-    mref_c = row_max_tail(mx, a0, mv0);  // O and l are still zero: nothing to rescale
+    float a0, mx = max16(sa);
+    row_max_exceeds(mx);
+    mref_c = move_reference(mx, a0);  // O and l are still zero: nothing to rescale
   }
   // step 0 sends K half tile 4 into the stage this S product has just read
   __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(63));

@@ -143,6 +143,31 @@ def test_bias_paths_agree(xmk):
     assert torch.equal(o1, o2)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_row_max_sees_every_key_of_a_tile(xmk, oracle, causal):
+    """A lane holds 16 of a half tile's 32 keys of its query row and gets the other 16 from lane l ^ 32.
+    Keys whose scores tower over the rest sit, in turn, in each of the two lanes' positions (key % 8 < 4
+    and >= 4) and only there: a row maximum that misses one lane's keys leaves the exponent reference
+    far below those scores and the exponentials overflow (raw score 1024, scaled 90.5: e^90 > fp32 max)."""
+    B, N, S, H = 1, 2, 256, 128
+    q = np.ones((B, N, S, H), dtype=np.float32)
+    v = oracle.normal((B, N, S, H), 77)
+    for upper in (0, 1):
+        k = np.zeros((B, N, S, H), dtype=np.float32)
+        big = (np.arange(S) % 8 >= 4) == bool(upper)
+        big[:40] = False  # the first steps set the reference from ordinary keys
+        k[:, :, big, :] = 8.0
+        qb, kb, vb = (oracle.from_f32(x, oracle.BF16) for x in (q, k, v))
+        out = torch.full((B, N, S, H), float("nan"), dtype=torch.bfloat16, device="cuda")
+        xmk.fmha_forward(to_dev(qb, "bf16"), to_dev(kb, "bf16"), to_dev(vb, "bf16"), out, causal=causal)
+        torch.cuda.synchronize()
+        got = out.float().cpu().numpy()
+        assert np.isfinite(got).all(), f"overflow with the large keys in lane half {upper}"
+        _, ref, _ = oracle.fmha_fwd(qb, kb, vb, oracle.BF16, H ** -0.5, causal=causal)
+        g, e = oracle.rel_err(got, ref.reshape(got.shape))
+        assert g <= 1e-2 and e <= 2e-2, (upper, g, e)
+
+
 def test_key_permutation_invariance(xmk):
     B, N, F, T, H = 1, 4, 256, 320, 128
     q = torch.randn((B, N, F, H), device="cuda").bfloat16()
