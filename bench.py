@@ -113,9 +113,10 @@ def gen(torch):
 
 
 class ClockSampler:
-    """Core clock (per XCD) and socket power as the SMI library reports them, read by a host thread
-    while a workload runs untimed: what the device held under that load, next to the published peak
-    (which assumes 2400 MHz).  Never running during a timed region."""
+    """Core clock (per XCD), socket power and throttler residencies as the SMI library reports them, read by
+    a host thread while a workload runs untimed: what the device held under that load, and which
+    limiter (package power tracking, thermal) held it there, next to the published peak (which
+    assumes 2400 MHz).  Never running during a timed region."""
 
     def __init__(self):
         self.smi = self.handle = None
@@ -152,12 +153,25 @@ class ClockSampler:
         except Exception:
             return None
 
+    THROTTLERS = ("ppt_residency_acc", "socket_thm_residency_acc", "vr_thm_residency_acc", "hbm_thm_residency_acc",
+                  "prochot_residency_acc")
+
+    def _residency(self):
+        """The firmware's accumulated throttler residencies and its sample counter (gpu_metrics)."""
+        try:
+            m = self.smi.amdsmi_get_gpu_metrics_info(self.handle)
+            out = {k: m.get(k) for k in self.THROTTLERS + ("accumulation_counter",)}
+            return out if all(isinstance(v, int) for v in out.values()) else None
+        except Exception:
+            return None
+
     def observe(self, torch, fn, seconds):
         """Runs fn back to back for `seconds` and samples every ~10 ms; returns the summary dict."""
         if self.smi is None or seconds <= 0:
             return {"source": self.source}
         import threading
         samples, stop = [], threading.Event()
+        res0 = None
 
         def loop():
             while not stop.is_set():
@@ -173,11 +187,13 @@ class ClockSampler:
                 fn()
             torch.cuda.synchronize()
             if not started and time.perf_counter() - t0 > 0.3 * seconds:  # sample the settled part only
+                res0 = self._residency() if self.metrics else None
                 th.start()
                 started = True
         stop.set()
         if started:
             th.join()
+        res1 = self._residency() if res0 else None
         if not samples:
             return {"source": self.source, "samples": 0}
         means = [sum(c) / len(c) for c, _ in samples]
@@ -187,11 +203,17 @@ class ClockSampler:
                "xcds": len(samples[0][0])}
         if pws:
             out["socket_power_w_mean"] = round(sum(pws) / len(pws))
+        if res0 and res1 and res1["accumulation_counter"] > res0["accumulation_counter"]:
+            # share of the firmware's samples in the window during which a throttler held the clock down
+            n = res1["accumulation_counter"] - res0["accumulation_counter"]
+            out["throttled"] = {k[:-len("_residency_acc")]: round((res1[k] - res0[k]) / n, 3) for k in self.THROTTLERS
+                                if res1[k] != res0[k]}
+            out["firmware_samples"] = n
         return out
 
 
 CLOCKS = None
-OBSERVE_SECONDS = 0.5
+OBSERVE_SECONDS = 1.0
 
 
 def _events(torch, fn, steps, warmup, graph=False):
@@ -554,7 +576,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--ramp", type=float, default=RAMP_SECONDS,
                     help="seconds of untimed launches before the warmup steps (0 for profiler runs)")
-    ap.add_argument("--observe", type=float, default=0.5,
+    ap.add_argument("--observe", type=float, default=1.0,
                     help="seconds each workload runs untimed, after its timed steps, while the SMI clocks are sampled "
                          "(0: no sampling, for profiler runs)")
     args = ap.parse_args()

@@ -12,9 +12,11 @@ namespace {
 template <typename T>
 void launch_t(const FmhaParams& p, int32_t dtype, uint64_t units, uint32_t F, bool causal, int bias, hipStream_t st) {
   // Head-size classes of the reference's policy choice (fmha_forward.h:622-646).  Four waves of 32
-  // query rows, two work-groups per CU: a second 32-row tile per wave (one wave per SIMD) was
-  // measured slower (741 against 796 TFLOP/s on [8,32,2048,128]), eight waves per work-group (half the
-  // K / V loads per row) equal, then and again on the current step (1020 against 1032).
+  // query rows, two work-groups per CU.  Measured against it on [8,32,2048,128] with the current step:
+  // eight waves per work-group (half the K / V loads per row) 1020 against 1032 TFLOP/s; a second
+  // 32-row tile per wave (one wave per SIMD, O in AGPRs, every K / V fragment feeding two matrix
+  // instructions) 1007 against 1033 without a mask and 789 against 872 with one, at a higher clock and
+  // the same board power and energy per launch: the package power limit, not the schedule, sets the rate.
   if (p.H <= 64) launch_cfg<T, 64, 4, 2>(p, units, F, causal, bias, st);
   else if (p.H <= 128) launch_cfg<T, 128, 4, 2>(p, units, F, causal, bias, st);
   else launch_h256(p, dtype, units, F, causal, bias, st);

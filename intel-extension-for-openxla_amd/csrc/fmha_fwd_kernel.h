@@ -471,39 +471,45 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
     // and it does not make the fragment reads wait for the loads in flight.
     [&](const char* __restrict__ knext, const char* __restrict__ vprev, char* __restrict__ kfree,
         char* __restrict__ vfree) {
+    // The step is written as a sequence of slots, one per matrix instruction, each closed by a
+    // scheduling fence: slot i sends the LDS fragment reads of matrix instruction i + D, issues matrix
+    // instruction i and runs its share of the vector work.  Empty asm statements pin every piece
+    // of vector work (its inputs at the start, its results at the end) and every accumulator to the
+    // slot, since arithmetic is otherwise free to drift across the fences.
+    constexpr int NS = sco ? KS : 0, NP = pv ? 2 * HT : 0, NM = NS + NP, D = kAhead;
+    constexpr int R0 = NS + 1, R1 = NS + 2;                   // slots of the row max of the new S
+    constexpr int NSLOT = sco ? (NM > R1 + 1 ? NM : R1 + 1) : (NM > 8 ? NM : 8);
+    const bool active = !masked || h - 1 < nh;
+    u32x4 frag[D + 1];
+    auto fetch = [&](auto I) {
+      constexpr int i = decltype(I)::value;
+      if constexpr (i < NS) {
+        frag[i % (D + 1)] = *reinterpret_cast<const u32x4*>(knext + kbase[i]);
+      } else if constexpr (i < NM) {
+        constexpr int q = i - NS, u = q / HT, ht = q % HT;
+        typedef short4v __attribute__((address_space(3))) * lds_ptr;
+        const char* vt = vprev + u * 16 * ROWB;
+        const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + vbase[ht][0]));
+        const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + vbase[ht][1]));
+        u32x4 vv;
+        vv[0] = __builtin_bit_cast(u32x2, lo)[0];
+        vv[1] = __builtin_bit_cast(u32x2, lo)[1];
+        vv[2] = __builtin_bit_cast(u32x2, hi)[0];
+        vv[3] = __builtin_bit_cast(u32x2, hi)[1];
+        frag[i % (D + 1)] = vv;
+      }
+    };
+    // The first fragment reads go out before the step's loads: sending the loads takes the wave about 170
+    // cycles, under which the reads' latency passes.
+    if (active) static_for<D>(fetch);
+    __builtin_amdgcn_sched_barrier(0);
     if (!masked || h + 4 < nhalf) issue_half(std::integral_constant<bool, !masked>{}, K, h + 4, kfree, koff, KV);
     if (!masked || h + 2 < nhalf) issue_half(std::integral_constant<bool, !masked>{}, V, h + 2, vfree, &voff, 1);
+    __builtin_amdgcn_sched_barrier(0);
     if constexpr ((HS & 1) == 1 && sco) take_bias((h + 1) / 2);
-    if (!masked || h - 1 < nh) {
+    if (active) {
       float alpha_n = 1.0f, mref_n = mref_c;
       bool moved_n = false;
-      // The step is written as a sequence of slots, one per matrix instruction, each closed by a
-      // scheduling fence: slot i sends the LDS fragment reads of matrix instruction i + D, issues matrix
-      // instruction i and runs its share of the vector work.  Empty asm statements pin every piece
-      // of vector work (its inputs at the start, its results at the end) and every accumulator to the
-      // slot, since arithmetic is otherwise free to drift across the fences.
-      constexpr int NS = sco ? KS : 0, NP = pv ? 2 * HT : 0, NM = NS + NP, D = kAhead;
-      constexpr int R0 = NS + 1, R1 = NS + 2;                   // slots of the row max of the new S
-      constexpr int NSLOT = sco ? (NM > R1 + 1 ? NM : R1 + 1) : (NM > 8 ? NM : 8);
-      u32x4 frag[D + 1];
-      auto fetch = [&](auto I) {
-        constexpr int i = decltype(I)::value;
-        if constexpr (i < NS) {
-          frag[i % (D + 1)] = *reinterpret_cast<const u32x4*>(knext + kbase[i]);
-        } else if constexpr (i < NM) {
-          constexpr int q = i - NS, u = q / HT, ht = q % HT;
-          typedef short4v __attribute__((address_space(3))) * lds_ptr;
-          const char* vt = vprev + u * 16 * ROWB;
-          const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + vbase[ht][0]));
-          const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(vt + vbase[ht][1]));
-          u32x4 vv;
-          vv[0] = __builtin_bit_cast(u32x2, lo)[0];
-          vv[1] = __builtin_bit_cast(u32x2, lo)[1];
-          vv[2] = __builtin_bit_cast(u32x2, hi)[0];
-          vv[3] = __builtin_bit_cast(u32x2, hi)[1];
-          frag[i % (D + 1)] = vv;
-        }
-      };
       auto fire = [&](auto I) {
         constexpr int i = decltype(I)::value;
         if constexpr (i < NS) {
@@ -546,7 +552,6 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
         moved_n = row_max_exceeds(mx);
         asm volatile("" : "+v"(mx));
       };
-      static_for<D>(fetch);
       static_for<NSLOT>([&](auto I) {
         constexpr int i = decltype(I)::value;
         fetch(std::integral_constant<int, i + D>{});

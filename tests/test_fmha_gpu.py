@@ -143,20 +143,22 @@ def test_bias_paths_agree(xmk):
     assert torch.equal(o1, o2)
 
 
+@pytest.mark.parametrize("H,big_k", [(64, 16.0), (128, 12.0), (256, 8.0)])
 @pytest.mark.parametrize("causal", [False, True])
-def test_row_max_sees_every_key_of_a_tile(xmk, oracle, causal):
+def test_row_max_sees_every_key_of_a_tile(xmk, oracle, causal, H, big_k):
     """A lane holds 16 of a half tile's 32 keys of its query row and gets the other 16 from lane l ^ 32.
     Keys whose scores tower over the rest sit, in turn, in each of the two lanes' positions (key % 8 < 4
     and >= 4) and only there: a row maximum that misses one lane's keys leaves the exponent reference
-    far below those scores and the exponentials overflow (raw score 1024, scaled 90.5: e^90 > fp32 max)."""
-    B, N, S, H = 1, 2, 256, 128
+    far below those scores and the exponentials overflow (scaled score 128 or more: e^128 > fp32 max).
+    Every head-size class of the kernel."""
+    B, N, S = 1, 2, 256
     q = np.ones((B, N, S, H), dtype=np.float32)
     v = oracle.normal((B, N, S, H), 77)
     for upper in (0, 1):
         k = np.zeros((B, N, S, H), dtype=np.float32)
         big = (np.arange(S) % 8 >= 4) == bool(upper)
         big[:40] = False  # the first steps set the reference from ordinary keys
-        k[:, :, big, :] = 8.0
+        k[:, :, big, :] = big_k
         qb, kb, vb = (oracle.from_f32(x, oracle.BF16) for x in (q, k, v))
         out = torch.full((B, N, S, H), float("nan"), dtype=torch.bfloat16, device="cuda")
         xmk.fmha_forward(to_dev(qb, "bf16"), to_dev(kb, "bf16"), to_dev(vb, "bf16"), out, causal=causal)
