@@ -23,13 +23,14 @@ RAMP_SECONDS = 0.25                                      # untimed launches befo
 
 # HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (KiB per dispatch), FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0: the factors a
-# 1 GiB device copy (--workload copy) gives on this machine.  The runs are summarised in
-# profiles/hbm_traffic_pmc.txt; a workload without a measurement reports null.
+# 1 GiB device copy (--workload copy) gives on this machine.  Counter figures of an earlier run of the same
+# kernels (profiles/hbm_traffic_pmc.txt says which build and when), not of the run that prints them: they are
+# to be measured again whenever one of these kernels changes.  A workload without a measurement reports null.
 TRAFFIC_BYTES = {
-    "fmha_causal": (224900 * 2.0 + 131100) * 1024,
-    "gemm_8192": (791700 * 2.0 + 131100) * 1024,
-    "int4_m1": (17480 * 2.0 + 32) * 1024,
-    "fp8_8192": (393600 * 2.0 + 131100) * 1024,
+    "fmha_causal": (221210 * 2.0 + 131070) * 1024,
+    "gemm_8192": (790500 * 2.0 + 131070) * 1024,
+    "int4_m1": (17487 * 2.0 + 32) * 1024,
+    "fp8_8192": (393620 * 2.0 + 131070) * 1024,
 }
 
 
@@ -186,7 +187,7 @@ class ClockSampler:
             for _ in range(8):
                 fn()
             torch.cuda.synchronize()
-            if not started and time.perf_counter() - t0 > 0.3 * seconds:  # sample the settled part only
+            if not started and time.perf_counter() - t0 > 0.5 * seconds:  # sample the settled part only
                 res0 = self._residency() if self.metrics else None
                 th.start()
                 started = True
