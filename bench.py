@@ -159,12 +159,16 @@ class ClockSampler:
 
     def _residency(self):
         """The firmware's accumulated throttler residencies and its sample counter (gpu_metrics)."""
-        try:
-            m = self.smi.amdsmi_get_gpu_metrics_info(self.handle)
-            out = {k: m.get(k) for k in self.THROTTLERS + ("accumulation_counter",)}
-            return out if all(isinstance(v, int) for v in out.values()) else None
-        except Exception:
-            return None
+        for _ in range(3):  # the call fails now and then while the device is busy
+            try:
+                m = self.smi.amdsmi_get_gpu_metrics_info(self.handle)
+                out = {k: m.get(k) for k in self.THROTTLERS + ("accumulation_counter",)}
+                if all(isinstance(v, int) for v in out.values()):
+                    return out
+            except Exception:
+                pass
+            time.sleep(0.002)
+        return None
 
     def observe(self, torch, fn, seconds):
         """Runs fn back to back for `seconds` and samples every ~10 ms; returns the summary dict."""
@@ -207,8 +211,7 @@ class ClockSampler:
         if res0 and res1 and res1["accumulation_counter"] > res0["accumulation_counter"]:
             # share of the firmware's samples in the window during which a throttler held the clock down
             n = res1["accumulation_counter"] - res0["accumulation_counter"]
-            out["throttled"] = {k[:-len("_residency_acc")]: round((res1[k] - res0[k]) / n, 3) for k in self.THROTTLERS
-                                if res1[k] != res0[k]}
+            out["throttled"] = {k[:-len("_residency_acc")]: round((res1[k] - res0[k]) / n, 3) for k in self.THROTTLERS}
             out["firmware_samples"] = n
         return out
 

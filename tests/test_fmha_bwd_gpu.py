@@ -2,14 +2,17 @@
 float64 closed form (pinned by finite differences in tests/test_oracle_math.py).
 
 Tolerance: error relative to the tensor's scale (oracle.rel_err's first figure) <= 1e-2 as for the
-forward outputs; the elementwise figure <= 1e-2 for fp16 and <= 8e-2 (eight times that: three
-mantissa bits fewer) for bf16.  P, dS and the forward output O (which enters through
-D = rowsum(dO o O)) are rounded to the 16-bit operand type before the products that consume them,
-here as in the reference (xetla/sdp/fmha_backward.h:195-196); the measured elementwise error is
-rounding-dominated: <= 0.4 % for fp16 and <= 5.4 % for bf16 (largest under a causal mask, where late
-keys receive few terms), the same for the fused kernels and for the GEMM
-composition (XMK_FMHA_BWD_COMPOSED=1, which test_backward_composition runs in a child process).  The reference's own attention test allows atol 3e-2 for
-bf16 and 1e-2 for fp16 on O(1) outputs (test/jax_ut.patch:997)."""
+forward outputs.  The elementwise figure (eps = rms(ref)) is held to 1e-2 for fp16 on every shape
+(measured maximum 3.9e-3) and, for bf16, to 1.5 times the measured maximum of each group of cases:
+8e-2 on the small shapes (measured 5.3e-2) and 1.5e-1 on the shapes with thousands of rows
+(measured 9.9e-2: the maximum over 1.5 M elements of a rounding-dominated error sits further out
+in the tail).  P, dS and the forward output O (which enters through D = rowsum(dO o O)) are rounded
+to the 16-bit operand type before the products that consume them, here as in the reference
+(xetla/sdp/fmha_backward.h:195-196); with three mantissa bits fewer than fp16 that rounding is the
+bf16 error, largest under a causal mask, where late keys receive few terms, and the same for the
+fused kernels and for the GEMM composition (XMK_FMHA_BWD_COMPOSED=1, which test_backward_composition
+runs in a child process).  The reference's own attention test allows atol 3e-2 for bf16 and 1e-2 for
+fp16 on O(1) outputs (test/jax_ut.patch:997)."""
 import numpy as np
 import pytest
 import torch
@@ -18,7 +21,8 @@ from util import to_dev
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
-TOL_ELEM = {"bf16": 8e-2, "fp16": 1e-2}
+TOL_ELEM = {"bf16": 8e-2, "fp16": 1e-2}        # small shapes
+TOL_ELEM_LARGE = {"bf16": 1.5e-1, "fp16": 1e-2}  # thousands of rows
 
 
 def _run(xmk, oracle, name, B, N, F, T, H, causal, use_bias, seed=0, tol_elem=None):
@@ -56,10 +60,8 @@ def test_backward_shapes(xmk, oracle, name, causal, use_bias, F, T, H):
 
 
 def test_backward_large(xmk, oracle):
-    """Many blocks with a bias and a causal mask.  The maximum over 1.5 M elements of a
-    rounding-dominated error sits further out in the tail than on the small shapes, so the
-    elementwise bound is wider here; the scale-relative bound is the same."""
-    errs = _run(xmk, oracle, "bf16", 1, 12, 2048, 2048, 64, True, True, seed=9, tol_elem=1e-1)
+    """Many blocks with a bias and a causal mask; the elementwise bound of the large shapes."""
+    errs = _run(xmk, oracle, "bf16", 1, 12, 2048, 2048, 64, True, True, seed=9, tol_elem=TOL_ELEM_LARGE["bf16"])
     print(errs)
 
 
@@ -73,7 +75,7 @@ xmk = importlib.import_module("intel-extension-for-openxla_amd")
 t._run(xmk, oracle, "fp16", 2, 3, 200, 136, 128, True, True)
 t._run(xmk, oracle, "bf16", 2, 3, 257, 64, 256, False, False)
 # more units than fit one workspace chunk (score buffers are capped at 1 GiB)
-t._run(xmk, oracle, "bf16", 1, 12, 2048, 2048, 64, True, False, seed=9, tol_elem=1e-1)
+t._run(xmk, oracle, "bf16", 1, 12, 2048, 2048, 64, True, False, seed=9, tol_elem=t.TOL_ELEM_LARGE["bf16"])
 print("composed ok")
 """
 
@@ -94,9 +96,8 @@ def test_backward_composition():
 @pytest.mark.parametrize("name,causal", [("bf16", True), ("fp16", False)])
 def test_backward_fused_long(xmk, oracle, name, causal):
     """The fused kernels over many blocks in both directions (16 key blocks, 8 owner blocks), ragged
-    ends in F and T; the elementwise bound is widened as for the other large case."""
-    errs = _run(xmk, oracle, name, 1, 3, 1000, 1016, 128, causal, False, seed=21,
-                tol_elem=1e-1 if name == "bf16" else 2e-2)
+    ends in F and T; the elementwise bound of the large shapes."""
+    errs = _run(xmk, oracle, name, 1, 3, 1000, 1016, 128, causal, False, seed=21, tol_elem=TOL_ELEM_LARGE[name])
     print(errs)
 
 
