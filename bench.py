@@ -171,12 +171,12 @@ class ClockSampler:
         return None
 
     def observe(self, torch, fn, seconds):
-        """Runs fn back to back for `seconds` and samples every ~10 ms; returns the summary dict."""
+        """Runs fn back to back for `seconds` (longer when the firmware's counters have not ticked twice by
+        then) and samples the clocks every ~10 ms; returns the summary dict."""
         if self.smi is None or seconds <= 0:
             return {"source": self.source}
         import threading
         samples, stop = [], threading.Event()
-        res0 = None
 
         def loop():
             while not stop.is_set():
@@ -185,20 +185,34 @@ class ClockSampler:
                     samples.append(r)
                 time.sleep(0.01)
         th = threading.Thread(target=loop, daemon=True)
+        # The firmware publishes its throttler residencies about once a second, 1000 samples at a time: a
+        # difference between two publications that both fall inside this run covers this workload only.
+        ticks = []
+        last = self._residency() if self.metrics else None
         t0 = time.perf_counter()
         started = False
-        while time.perf_counter() - t0 < seconds:
-            for _ in range(8):
+        burst = 8
+        while True:
+            tb = time.perf_counter()
+            for _ in range(burst):
                 fn()
             torch.cuda.synchronize()
-            if not started and time.perf_counter() - t0 > 0.5 * seconds:  # sample the settled part only
-                res0 = self._residency() if self.metrics else None
+            el = time.perf_counter() - t0
+            # bursts of about 25 ms, so that the host's reads between them leave the device busy
+            burst = max(8, min(4096, int(burst * 0.025 / max(time.perf_counter() - tb, 1e-5))))
+            if last is not None:
+                r = self._residency()
+                if r and r["accumulation_counter"] != last["accumulation_counter"]:
+                    ticks.append(r)
+                    last = r
+            if not started and el > 0.5 * seconds:  # clocks: the settled part only
                 th.start()
                 started = True
+            if el >= seconds and (last is None or len(ticks) >= 2 or el >= seconds + 1.5):
+                break
         stop.set()
         if started:
             th.join()
-        res1 = self._residency() if res0 else None
         if not samples:
             return {"source": self.source, "samples": 0}
         means = [sum(c) / len(c) for c, _ in samples]
@@ -208,11 +222,13 @@ class ClockSampler:
                "xcds": len(samples[0][0])}
         if pws:
             out["socket_power_w_mean"] = round(sum(pws) / len(pws))
-        if res0 and res1 and res1["accumulation_counter"] > res0["accumulation_counter"]:
-            # share of the firmware's samples in the window during which a throttler held the clock down
-            n = res1["accumulation_counter"] - res0["accumulation_counter"]
-            out["throttled"] = {k[:-len("_residency_acc")]: round((res1[k] - res0[k]) / n, 3) for k in self.THROTTLERS}
-            out["firmware_samples"] = n
+        if len(ticks) >= 2:
+            # share of the firmware's samples between two publications during which a throttler held the clock down
+            n = ticks[-1]["accumulation_counter"] - ticks[0]["accumulation_counter"]
+            if n > 0:
+                out["throttled"] = {k[:-len("_residency_acc")]: round((ticks[-1][k] - ticks[0][k]) / n, 3)
+                                    for k in self.THROTTLERS}
+                out["firmware_samples"] = n
         return out
 
 
