@@ -14,6 +14,7 @@
 // is bound by HBM only if the per-weight VALU work stays near one operation, so the
 // nibbles are expanded with the fp16 "magic number" trick (5 operations per 8 weights).
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.h"
 #include "int4_gemm.h"
@@ -57,12 +58,13 @@ __device__ __forceinline__ half8 unpack_word(uint32_t w, uint32_t m1024, uint32_
 }
 
 // 8 consecutive activations -> the same k-slot order (0,4,1,5,2,6,3,7).
-__device__ __forceinline__ half8 permute_act(u32x4 d) {
+// sel_lo = 0x05040100, sel_hi = 0x07060302 (passed in so that the caller can order these operations).
+__device__ __forceinline__ half8 permute_act(u32x4 d, uint32_t sel_lo, uint32_t sel_hi) {
   Frag f;
-  f.u[0] = __builtin_amdgcn_perm(d[2], d[0], 0x05040100u);  // (h0, h4)
-  f.u[1] = __builtin_amdgcn_perm(d[2], d[0], 0x07060302u);  // (h1, h5)
-  f.u[2] = __builtin_amdgcn_perm(d[3], d[1], 0x05040100u);  // (h2, h6)
-  f.u[3] = __builtin_amdgcn_perm(d[3], d[1], 0x07060302u);  // (h3, h7)
+  f.u[0] = __builtin_amdgcn_perm(d[2], d[0], sel_lo);  // (h0, h4)
+  f.u[1] = __builtin_amdgcn_perm(d[2], d[0], sel_hi);  // (h1, h5)
+  f.u[2] = __builtin_amdgcn_perm(d[3], d[1], sel_lo);  // (h2, h6)
+  f.u[3] = __builtin_amdgcn_perm(d[3], d[1], sel_hi);  // (h3, h7)
   return f.h;
 }
 
@@ -140,6 +142,14 @@ struct Int4Problem {
   float* partial;
 };
 
+// f(integral_constant<I>), ..., f(integral_constant<N - 1>) in turn, stopping after the first that returns false.
+template <int I, int N, class F>
+__device__ __forceinline__ void static_steps(F&& f) {
+  if constexpr (I < N) {
+    if (f(std::integral_constant<int, I>{})) static_steps<I + 1, N>(f);
+  }
+}
+
 template <int W, int MT, int RI, int SPG, int NW, bool SK, bool SPREAD, int SDIV = 1>
 __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0, int mixed) {
   // mixed (two K-split products of equal width): the products alternate from one block to the next, and
@@ -212,24 +222,46 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     Words<(W + 1) / 2> sc, zp;
     u32x4 a[SPG][MT];
   };
-  auto fetch = [&](int g, GroupData& d) {
+  // kExact (eight-wave work-groups that own their whole reduction): a fetch past the wave's last group is
+  // still issued, with every lane out of range (no memory access, zeros returned), and the groups run as
+  // straight-line code, so that the sequence of loads is the same on every path and the counted waits
+  // the compiler places before a group's arithmetic leave the next group's loads in flight.  The other
+  // shapes keep a loop with fetches behind branches, whose waits drain the prefetch at every turn: measured
+  // on one device, the exact form is 9-12 % faster at 8 rows and 5 % at 32 (k 4096, n 16384), 3-5 % slower on
+  // the sixteen-wave one-row kernel and 1.4 % slower over a decode step (four-wave and K-split launches).
+  constexpr bool kExact = NW == 8 && !SK;
+  auto fetch = [&](int g, GroupData& d, bool live) {
     // (wave-uniform; said explicitly, or the compiler wraps each of the two loads in a loop over lane values)
     const uint32_t so = __builtin_amdgcn_readfirstlane((uint32_t)((g / SDIV) * N * 2));
-    d.sc = load_halves<W>(r_s, voff_sz, so);
-    d.zp = load_halves<W>(r_z, voff_sz, so);
+    const uint32_t vsz = live ? voff_sz : kOob, vw = live ? voff_w : kOob;
+    constexpr bool kPinned = kExact;
+    if constexpr (kPinned) __builtin_amdgcn_sched_barrier(0);  // the loads stay together and in this order
+    d.sc = load_halves<W>(r_s, vsz, so);
+    d.zp = load_halves<W>(r_z, vsz, so);
 #pragma unroll
     for (int s = 0; s < SPG; ++s)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
         d.a[s][mt] = __builtin_bit_cast(
-            u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_a, voff_a[mt], (uint32_t)((g * SPG + s) * 64), 0));
+            u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_a, live ? voff_a[mt] : kOob, (uint32_t)((g * SPG + s) * 64), 0));
 #pragma unroll
     for (int s = 0; s < SPG; ++s)
-      d.w[s] = load_words<W>(r_w, voff_w, (uint32_t)((g * 4 * SPG + s * 4) * N * 4));
+      d.w[s] = load_words<W>(r_w, vw, (uint32_t)((g * 4 * SPG + s * 4) * N * 4));
+    // Every unpack reads these constants and every activation shuffle a selector derived from them, so
+    // the arithmetic that follows in program order is also emitted after these loads (instruction
+    // selection is free to order what has no side effects, and would otherwise wait for a group's
+    // activations before the next fetch goes out).
+    if constexpr (kPinned) {
+      asm volatile("" : "+v"(m1024), "+v"(m64) : : "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
   auto compute = [&](const GroupData& cur) {
     floatx4 d[MT][W], asum[MT], noff[MT];
     half8 a[SPG][MT];
+    // (kExact: derived from the constant that the fetch has just laundered, see there)
+    const uint32_t sel_lo = kExact ? m64 ^ (0x54005400u ^ 0x05040100u) : 0x05040100u;
+    const uint32_t sel_hi = kExact ? m64 ^ (0x54005400u ^ 0x07060302u) : 0x07060302u;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       asum[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -241,7 +273,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     for (int s = 0; s < SPG; ++s)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        a[s][mt] = permute_act(cur.a[s][mt]);
+        a[s][mt] = permute_act(cur.a[s][mt], sel_lo, sel_hi);
         noff[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s][mt], noffs.h, noff[mt], 0, 0, 0);
       }
 #pragma unroll
@@ -271,20 +303,53 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     }
   };
 
-  GroupData bufA, bufB;  // ping-pong: no register copies between iterations
+  // Two register buffers, one group in flight while one is computed.  (Three were slower wherever they were
+  // tried: 5-7 % at 2 to 16 rows on the eight-wave form, 1.747 against 1.704 ms over a decode step on the
+  // four-wave one.)
+  constexpr int DEPTH = 2;
+  GroupData buf[DEPTH];
   // This work-group's share of the groups: all of them, or slice blockIdx.y of gridDim.y.
   const int gper = SK ? (ngroups + (int)gridDim.y - 1) / (int)gridDim.y : ngroups;
   const int gend = SK ? min(ngroups, ((int)blockIdx.y + 1) * gper) : ngroups;
-  int g = (SK ? (int)blockIdx.y * gper : 0) + wave;
-  if (g < gend) fetch(g, bufA);
-  while (g < gend) {
-    if (g + NW < gend) fetch(g + NW, bufB);
-    compute(bufA);
-    g += NW;
-    if (g >= gend) break;
-    if (g + NW < gend) fetch(g + NW, bufA);
-    compute(bufB);
-    g += NW;
+  int g = (SK ? (int)blockIdx.y * gper : 0) + wave;  // groups g, g + NW, ... below gend are this wave's
+  if constexpr (kExact) {
+    // The first kStraight groups as straight-line code with forward exits only: no loop edge merges two
+    // histories of outstanding loads.  (Around a loop with an exit in its middle the compiler's wait
+    // accounting merges the path that leaves with the path that goes round.)  Compile-time buffer indices
+    // throughout: a buffer indexed by a loop variable would live in scratch memory.
+    const int mine = g < gend ? (gend - g + NW - 1) / NW : 0;
+    constexpr int kStraight = DEPTH == 3 ? 9 : 8;
+    static_steps<0, DEPTH - 1>([&](auto j) {
+      fetch(g + j * NW, buf[j], j < mine);
+      return true;
+    });
+    static_steps<0, kStraight>([&](auto i) {
+      if (i >= mine) return false;
+      fetch(g + (i + DEPTH - 1) * NW, buf[(i + DEPTH - 1) % DEPTH], i + DEPTH - 1 < mine);
+      compute(buf[i % DEPTH]);
+      return true;
+    });
+    // long reductions: the rest in a loop (buf[j] holds group kStraight + j; kStraight is a multiple of DEPTH)
+    for (int i = kStraight; i < mine;) {
+      static_steps<0, DEPTH>([&](auto j) {
+        if (i >= mine) return false;
+        fetch(g + (i + DEPTH - 1) * NW, buf[(j + DEPTH - 1) % DEPTH], i + DEPTH - 1 < mine);
+        compute(buf[j]);
+        ++i;
+        return true;
+      });
+    }
+  } else {
+    if (g < gend) fetch(g, buf[0], true);
+    while (g < gend) {
+      if (g + NW < gend) fetch(g + NW, buf[1], true);
+      compute(buf[0]);
+      g += NW;
+      if (g >= gend) break;
+      if (g + NW < gend) fetch(g + NW, buf[0], true);
+      compute(buf[1]);
+      g += NW;
+    }
   }
 
   // Lane holds rows 4*kg+i (+16 mt) of columns col16*W+c.

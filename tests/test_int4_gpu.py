@@ -65,6 +65,9 @@ def test_int4_gemm_gptj_mlp_shape(xmk, oracle, m):
     (20, 256, 72, 128, False),      # fewer groups than waves
     (31, 640, 136, 128, True),      # 5 groups: waves with one group and waves with none
     (48, 4096, 1024, 128, True),    # 32 rows + 16 in a second launch
+    # more than eight groups per wave: the straight-line part is followed by the loop, which ends on an
+    # odd count (9 and 11 groups per wave) and after one group of the loop (9)
+    (10, 9216, 264, 128, True), (5, 5632, 136, 64, False), (30, 9216, 72, 128, False),
     # groups of 256 channels run as two batches of 128 with the same scale and zero point
     (1, 2048, 512, 256, True), (8, 1024, 264, 256, False), (32, 4096, 256, 256, True), (4, 4096, 4096, 256, False),
 ])
