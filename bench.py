@@ -103,13 +103,32 @@ class Seeded:
         return out.view(shape)
 
 
+class Constant:
+    """--data constant: every operand element the same value.  Not a benchmark input: with nothing toggling in
+    the operand paths the same kernels draw 150-300 W less and the device holds its full clock, so the run
+    shows what the schedule alone sustains, beside what the power limit leaves of it on the seeded data."""
+
+    def __init__(self, torch):
+        self.t = torch
+
+    def normal(self, shape, seed, scale=1.0, dtype=None):
+        return self.t.full(shape, 0.03125 * float(scale), dtype=dtype or self.t.float32, device="cuda")
+
+    def uniform(self, shape, seed, lo_v, hi_v, dtype=None):
+        return self.t.full(shape, 0.5 * (lo_v + hi_v), dtype=dtype or self.t.float32, device="cuda")
+
+    def words(self, shape, seed):
+        return self.t.full(shape, 0x11111111, dtype=self.t.int32, device="cuda")
+
+
 _GEN = None
+DATA = "seeded"
 
 
 def gen(torch):
     global _GEN
     if _GEN is None:
-        _GEN = Seeded(torch)
+        _GEN = Constant(torch) if DATA == "constant" else Seeded(torch)
     return _GEN
 
 
@@ -599,6 +618,9 @@ def main():
     ap.add_argument("--observe", type=float, default=1.0,
                     help="seconds each workload runs untimed, after its timed steps, while the SMI clocks are sampled "
                          "(0: no sampling, for profiler runs)")
+    ap.add_argument("--data", default="seeded", choices=["seeded", "constant"],
+                    help="seeded: the parity tests' generator (the benchmark); constant: every operand element equal "
+                         "(a power experiment: see class Constant)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1",
@@ -606,6 +628,7 @@ def main():
         sys.exit(2)
 
     globals()["RAMP_SECONDS"] = args.ramp
+    globals()["DATA"] = args.data
     import torch
     xmk = importlib.import_module("intel-extension-for-openxla_amd")
     xmk.lib()  # fails loudly if libxmk.so is missing: there is no fallback path
@@ -619,7 +642,8 @@ def main():
         "metric": "TFLOP/s & %MFMA peak (GEMM/MHA); int4 GEMV HBM GB/s & %peak; 1 GPU",
         "value": roof["achieved"], "unit": roof["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"],
+        "data": "synthetic" if args.data == "seeded" else "synthetic, constant operands (power experiment, not a benchmark figure)",
         "config": {"workload": w["name"], "note": w.get("note", "")},
         "roofline": roof,
     }
