@@ -388,7 +388,8 @@ def wl_gemv_f16(torch, xmk, m=1, n=16384, k=4096, copies=4):
         state[0] += 1
         xmk.run_gemm(a, b, out, workspace=ws)
     return dict(name=f"gemm_f16_m{m}_n{n}_k{k}", fn=fn, flops=2.0 * m * n * k, bytes=2.0 * (m * k + k * n + m * n),
-                bound="hbm", dtype="f16", kernel="gemm_mfma_kernel (+ splitk_reduce_kernel)", graph=True,
+                bound="hbm", dtype="f16", graph=True,
+                kernel=xmk.gemm_policy_name(m, n, k, False, xmk.F16, xmk.F16) + (" + splitk_reduce_kernel" if need else ""),
                 note=f"xmk_gemm_ws, {need} bytes of K-split scratch" if need else "xmk_gemm, unsplit")
 
 

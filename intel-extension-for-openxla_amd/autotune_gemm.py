@@ -23,8 +23,11 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 TABLE = os.path.join(HERE, "csrc", "gemm_policy_table.h")
 POLICIES = ["mfma_256x256x32_w2x2_s4", "mfma_128x128x64_w2x2_s3", "mfma_128x64x64_w2x2_s4", "mfma_64x64x64_w2x2_s4",
-            "mfma_256x128x64_w2x2_s3"]
-TILES = [(256, 256), (128, 128), (128, 64), (64, 64), (256, 128)]
+            "mfma_256x128x64_w2x2_s3", "stream_rows_8x512_w8"]
+TILES = [(256, 256), (128, 128), (128, 64), (64, 64), (256, 128)]  # the matrix-core policies (the heuristic's candidates)
+# The last policy is the streaming kernel for up to eight rows: forced on a shape it cannot take, the library
+# falls back to its own choice, so such a candidate simply repeats the default's time.
+MFMA_POLICIES = len(TILES)
 
 # (n, k) pairs of the reference's LLM shape list (gemm.cc:31-285) that fit the medium/large-M tiles,
 # plus the benchmark shapes.
@@ -145,7 +148,9 @@ def tune_small(shapes, args):
     rows = load_table()
     for (m, n, k) in shapes:
         key = f"{m},{n},{k}"
-        best = min(cand, key=lambda c: cand[c][key])
+        # (the streaming kernel takes at most eight rows: with more, that candidate only repeats the default)
+        usable = [c for c in cand if c[0] < MFMA_POLICIES or m <= 8]
+        best = min(usable, key=lambda c: cand[c][key])
         t0, t1 = base[key] * 1e3, cand[best][key] * 1e3
         gbs = 2.0 * (m * k + k * n + m * n) / t0 / 1e3
         print(f"{key:>18}: default {t0:7.2f} us ({gbs:5.0f} GB/s)  best {t1:7.2f} us  = {POLICIES[best[0]]} x {best[1]} slices")
@@ -202,13 +207,13 @@ def main():
         tune_small(shapes, args)
         return
     times = []
-    for pol in range(len(POLICIES)):
+    for pol in range(MFMA_POLICIES):
         times.append(run_worker(shapes, {"XMK_GEMM_POLICY": str(pol)}, "--worker"))
         print(f"policy {pol} ({POLICIES[pol]}) measured", flush=True)
     rows = []
     for (m, n, k) in shapes:
         key = f"{m},{n},{k}"
-        t = [times[p][key] for p in range(len(POLICIES))]
+        t = [times[p][key] for p in range(MFMA_POLICIES)]
         best, h = min(range(len(t)), key=lambda i: t[i]), heuristic(m, n, k)
         tf = [2.0 * m * n * k / x / 1e9 for x in t]
         print(f"{key:>18}: " + " ".join(f"{x:7.1f}" for x in tf) + f"  TFLOP/s  heuristic {h} best {best}")

@@ -23,6 +23,7 @@
 // the reference falls back to oneDNN (onednn_matmul_utils.cc:394-491).
 #include "gemm_f32.h"
 #include "gemm_kernel.h"
+#include "gemm_rows.h"
 #include "gemm_s8.h"
 
 namespace {
@@ -193,18 +194,38 @@ int elem_size(int dtype) {
 
 extern "C" const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int32_t rhs_transpose,
                                             int32_t dtype_in, int32_t dtype_out) {
-  (void)rhs_transpose;
   const bool sixteen = dtype_in == XMK_BF16 || dtype_in == XMK_F16;
   if (dtype_in == XMK_F32 && dtype_out == XMK_F32) return "mfma_f32_128x128x16";
   if (dtype_in == XMK_S8 && dtype_out == XMK_S32) return "mfma_s8_128x128x64";
   if (!sixteen || !(dtype_out == dtype_in || dtype_out == XMK_F32)) return "generic_64x64";
-  return kPolicies[select_policy(m, n, k)].name;
+  // (packed, aligned operands assumed, as everywhere in this query)
+  const bool rows_ok = !rhs_transpose && m >= 1 && m <= kRowsMaxM && n % 8 == 0 && k % 8 == 0;
+  return kPolicies[select_policy(m, n, k, 1, rows_ok)].name;
 }
 
 namespace {
 // out1 / out2: further outputs of the shared-lhs three-GEMM form, or null for a plain GEMM.
 // policy: tile policy to use instead of select_policy's choice (the K-split planner's), or -1.
 int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int policy = -1);
+
+// The conditions of the direct (non-gathering) 16-bit kernels on the stored operands.
+bool direct_ok(const xmk_matrix& lhs, const xmk_matrix& rhs) {
+  return xmk::aligned(lhs.data, 16) && xmk::aligned(rhs.data, 16) && lhs.leading_dim_stride % 8 == 0 &&
+         rhs.leading_dim_stride % 8 == 0 && lhs.batch_stride % 8 == 0 && rhs.batch_stride % 8 == 0 &&
+         lhs.num_cols % 8 == 0 && rhs.num_cols % 8 == 0;
+}
+
+// Whether the streaming kernel for a few rows (gemm_rows.hip) can run this descriptor's product.
+bool rows_ok_desc(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k) {
+  if (d->out.transpose || d->lhs.transpose || d->rhs.transpose || !direct_ok(d->lhs, d->rhs) ||
+      !xmk::aligned(d->out.data, 16))
+    return false;
+  if (d->dtype_in != XMK_BF16 && d->dtype_in != XMK_F16) return false;
+  GemmParams p{};
+  p.M = (int)m; p.N = (int)n; p.K = (int)k;
+  p.lda = d->lhs.leading_dim_stride; p.ldb = d->rhs.leading_dim_stride;
+  return gemm_rows_applicable(p, false, true);
+}
 
 // K slices worth using for a plain 16-bit GEMM of this shape when scratch is available: few
 // output tiles (the device has 256 CUs) and a long reduction.  1: do not split.
@@ -218,9 +239,22 @@ int plan_splitk(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k, int* po
   const char* forced_env = getenv("XMK_GEMM_SPLITK");
   const int forced = forced_env ? atoi(forced_env) : 0;
   if (forced >= 1) return divides(forced) ? forced : 1;
-  if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit >= 1 && divides(t->ksplit)) {
+  const bool rows_ok = rows_ok_desc(d, m, n, k) && (forced_policy() < 0 || forced_policy() == kRowsPolicy);
+  if (const TunedShape* t = tuned_shape(m, n, k); forced_policy() < 0 && t && t->ksplit >= 1 && divides(t->ksplit) &&
+                                                  (t->policy != kRowsPolicy || rows_ok)) {
     if (t->ksplit > 1) *policy = t->policy;
     return t->ksplit;
+  }
+  if (rows_ok && xmk::ceil_div(n, (int64_t)kRowsDefaultBN) >= kRowsEnoughBlocks) return 1;  // streamed in one launch
+  if (rows_ok && forced_policy() == kRowsPolicy) {
+    // The streaming kernel forced on a narrower matrix (tests, the autotuner): slices until its narrowest
+    // column blocks are about one work-group per CU, each slice keeping 512 rows (a batch of 64 per wave).
+    const int64_t blocks = xmk::ceil_div(n, (int64_t)kRowsMinBN);
+    int ks = 1;
+    if (blocks < kRowsEnoughBlocks)
+      while (ks < 16 && blocks * ks < 256 && k % (ks * 2 * 8) == 0 && k / (ks * 2) >= 512) ks *= 2;
+    if (ks > 1) *policy = kRowsPolicy;
+    return ks;
   }
   const Policy& pol = kPolicies[select_policy(m, n, k)];
   const int64_t tiles = xmk::ceil_div(m, pol.bm) * xmk::ceil_div(n, pol.bn);
@@ -387,11 +421,8 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int p
   hipStream_t st = (hipStream_t)stream;
   const bool qkv = out1 != nullptr;
   const bool sixteen = din == XMK_BF16 || din == XMK_F16;
-  const bool fast = sixteen && xmk::aligned(lhs.data, 16) && xmk::aligned(rhs.data, 16) &&
-                    xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) && xmk::aligned(out2, 16) &&
-                    lhs.leading_dim_stride % 8 == 0 &&
-                    rhs.leading_dim_stride % 8 == 0 && lhs.batch_stride % 8 == 0 &&
-                    rhs.batch_stride % 8 == 0 && lhs.num_cols % 8 == 0 && rhs.num_cols % 8 == 0;
+  const bool fast = sixteen && direct_ok(lhs, rhs) && xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) &&
+                    xmk::aligned(out2, 16);
   // 16-bit operands that miss those conditions still run on the matrix cores, with operands gathered
   // element by element; the output pointers must allow the epilogue's vector stores.
   const bool gather = !fast && sixteen && xmk::aligned(out.data, 16) && xmk::aligned(out1, 16) &&
@@ -419,7 +450,10 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int p
     const bool a_mc = lhs.transpose != 0;   // stored [K, M]
     const bool b_mc = rhs.transpose == 0;   // stored [K, N]
     const int batch = qkv ? 3 : (int)d->batch_size;
-    const int pol = (policy >= 0 && policy < kNumPolicies) ? policy : select_policy(m, n, k, batch);
+    const bool rows_ok = fast && gemm_rows_applicable(p, a_mc, b_mc);
+    // the forced policy first, then the K-split planner's, then the table and the rules
+    const int pol = (forced_policy() < 0 && policy >= 0 && policy < kNumPolicies && (policy != kRowsPolicy || rows_ok))
+                        ? policy : select_policy(m, n, k, batch, rows_ok);
     xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s",
                (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
                rhs.transpose, d->epilogue, d->beta, gather ? kGatherPolicy.name : kPolicies[pol].name);
@@ -431,6 +465,10 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int p
         if (dout == XMK_F32) launch_layout_gather<_Float16, true>(a_mc, b_mc, p, batch, st);
         else launch_layout_gather<_Float16, false>(a_mc, b_mc, p, batch, st);
       }
+      return xmk::check_launch("gemm");
+    }
+    if (pol == kRowsPolicy) {
+      launch_gemm_rows(p, din == XMK_BF16, dout == XMK_F32, batch, st);
       return xmk::check_launch("gemm");
     }
     if (din == XMK_BF16) {

@@ -653,8 +653,21 @@ constexpr Policy kPolicies[] = {
     {"mfma_128x64x64_w2x2_s4", 128, 64, 2, 2, 64, 4},
     {"mfma_64x64x64_w2x2_s4", 64, 64, 2, 2, 64, 4},
     {"mfma_256x128x64_w2x2_s3", 256, 128, 2, 2, 64, 3},
+    // not a matrix-core tile: the streaming kernel for up to eight rows (gemm_rows.hip), eight waves
+    // that split the reduction of a 512-column block
+    {"stream_rows_8x512_w8", 8, 512, 8, 1, 8, 2},
 };
 constexpr int kNumPolicies = sizeof(kPolicies) / sizeof(kPolicies[0]);
+constexpr int kRowsPolicy = kNumPolicies - 1;
+constexpr int kRowsMaxM = 8;            // rows the streaming kernel takes
+constexpr int kRowsMinBN = 64;          // its output columns per work-group: 64, 128, 256 or 512
+constexpr int kRowsEnoughBlocks = 192;  // work-groups from which on a launch pulls the memory system's rate
+// The streaming kernel is the default where 128-column blocks are already that many work-groups, i.e. from
+// 24.5 thousand columns on (the vocabulary projections).  Measured, fp16, k = 4096, microseconds, best
+// matrix-core choice against best streaming choice: n = 50400, m = 4: 96.9 / 71.9 (5.75 TB/s); n = 16384,
+// m = 1: 27.7 / 28.5, m = 4: 27.4 / 31.1; n = 12288, m = 8: 25.9 / 32.2; n = 4096, k = 16384, m = 4:
+// 30.1 / 36.8: below that width a launch is over before the stream has paid for its start and end.
+constexpr int kRowsDefaultBN = 128;
 
 // Tile choice, the role of selectXetlaGemmConfig (xetla/gemm/gemm.cc:286-308).  Shapes listed in the tuned table
 // (gemm_policy_table.h, written by autotune_gemm.py from measurements) take the policy
@@ -671,22 +684,30 @@ inline const TunedShape* tuned_shape(int64_t m, int64_t n, int64_t k) {
     if (t.m == m && t.n == n && t.k == k) return &t;
   return nullptr;
 }
-inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1) {
-  // read at every call (a getenv costs far less than a launch), so that the autotuner can walk the
-  // policies inside one process
+// XMK_GEMM_POLICY=<index>, or -1.  Read at every call (a getenv costs far less than a launch), so that the
+// autotuner can walk the policies inside one process.
+inline int forced_policy() {
   if (const char* e = getenv("XMK_GEMM_POLICY")) {
     const int v = atoi(e);
     if (*e && v >= 0 && v < kNumPolicies) return v;
   }
+  return -1;
+}
+// rows_ok: the operands meet the streaming kernel's conditions (gemm_rows_applicable); it is never chosen otherwise.
+inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1, bool rows_ok = false) {
+  auto usable = [&](int v) { return v >= 0 && v < kNumPolicies && (v != kRowsPolicy || rows_ok); };
+  if (const int v = forced_policy(); usable(v)) return v;
   if (batch == 1)
-    if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit <= 1) return t->policy;
+    if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit <= 1 && usable(t->policy)) return t->policy;
+  // A few rows against a very wide matrix: stream it.
+  if (rows_ok && batch == 1 && xmk::ceil_div(n, kRowsDefaultBN) >= kRowsEnoughBlocks) return kRowsPolicy;
   // Heuristic: the policy with the best estimated throughput = (what the tile sustains when the
   // device is full) x (share of the 256 CUs busy over the tile waves) x (share of the tiles' area
   // inside the matrix).  The per-tile figures are measured large-shape rates relative to 256x256.
-  static constexpr float kTileRate[kNumPolicies] = {1.0f, 0.75f, 0.60f, 0.55f, 0.90f};
-  int best = kNumPolicies - 1;
+  static constexpr float kTileRate[kRowsPolicy] = {1.0f, 0.75f, 0.60f, 0.55f, 0.90f};
+  int best = kRowsPolicy - 1;
   float best_score = -1.0f;
-  for (int i = 0; i < kNumPolicies; ++i) {
+  for (int i = 0; i < kRowsPolicy; ++i) {
     const int64_t tiles = xmk::ceil_div(m, kPolicies[i].bm) * xmk::ceil_div(n, kPolicies[i].bn) * batch;
     const int64_t waves = xmk::ceil_div(tiles, 256);
     const float busy = (float)tiles / (float)(waves * 256);
