@@ -89,16 +89,19 @@ __global__ __launch_bounds__(kNW * 64) void gemm_rows_kernel(GemmParams p) {
   auto fetch = [&](int q, Chunk& c) {
     const bool live = 8 * (G * q + g) < p.K;  // K % 8 == 0: a lane's eight rows are all in or all out
     const uint32_t vb = live ? voff_b : kOob;
+    // (a batch wholly past the end uses batch 0's scalar offsets, so that kOob plus the scalar offset cannot
+    //  wrap around 32 bits whatever the unit that checks the range adds up)
+    const int64_t qs = 8 * G * q < p.K ? q : 0;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < MT; ++m)
       c.a[m] = __builtin_bit_cast(
           u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_a, (live && m < p.M) ? voff_a : kOob,
-                                                       (uint32_t)(((int64_t)m * p.lda + (int64_t)q * 8 * G) * 2), 0));
+                                                       (uint32_t)(((int64_t)m * p.lda + qs * 8 * G) * 2), 0));
 #pragma unroll
     for (int j = 0; j < kChunk; ++j)
       c.b[j] = __builtin_bit_cast(
-          u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_b, vb, (uint32_t)(((int64_t)q * 8 * G + j) * p.ldb * 2), 0));
+          u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_b, vb, (uint32_t)((qs * 8 * G + j) * p.ldb * 2), 0));
     // Every pairing below reads these selectors, so the arithmetic that follows in program order is also
     // emitted after these loads (instruction selection is free to order what has no side effects).
     asm volatile("" : "+v"(sel_lo), "+v"(sel_hi) : : "memory");
@@ -208,7 +211,8 @@ bool gemm_rows_applicable(const GemmParams& p, bool a_mc, bool b_mc) {
   if (a_mc || !b_mc || p.M < 1 || p.M > kRowsMaxM || p.N % 8 != 0 || p.K % kChunk != 0) return false;
   if (p.out_alt[0] || p.out_alt[1]) return false;
   constexpr int64_t kLimit = int64_t{1} << 31;  // byte offsets below kOob
-  return ((int64_t)(p.K - 1) * p.ldb + p.N) * 2 < kLimit && ((int64_t)(p.M - 1) * p.lda + p.K) * 2 < kLimit;
+  // (a wave's batch is up to 64 rows, the last of which may lie past K)
+  return ((int64_t)(p.K + 63) * p.ldb + p.N) * 2 < kLimit && ((int64_t)(p.M - 1) * p.lda + p.K + 64) * 2 < kLimit;
 }
 
 void launch_gemm_rows(const GemmParams& p, bool is_bf16, bool out_f32, int batch, hipStream_t st) {

@@ -230,7 +230,10 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   // on one device, the exact form is 9-12 % faster at 8 rows and 5 % at 32 (k 4096, n 16384), 3-5 % slower on
   // the sixteen-wave one-row kernel and 1.4 % slower over a decode step (four-wave and K-split launches).
   constexpr bool kExact = NW == 8 && !SK;
-  auto fetch = [&](int g, GroupData& d, bool live) {
+  auto fetch = [&](int g_asked, GroupData& d, bool live) {
+    // (a fetch past the end uses group 0's scalar offsets, so that kOob plus the scalar offset cannot wrap
+    //  around 32 bits whatever the unit that checks the range adds up)
+    const int g = live ? g_asked : 0;
     // (wave-uniform; said explicitly, or the compiler wraps each of the two loads in a loop over lane values)
     const uint32_t so = __builtin_amdgcn_readfirstlane((uint32_t)((g / SDIV) * N * 2));
     const uint32_t vsz = live ? voff_sz : kOob, vw = live ? voff_w : kOob;
