@@ -371,26 +371,26 @@ def wl_int4(torch, xmk, m, k=4096, n=16384, group=128, copies=12):
                 bound="hbm", dtype="f16", kernel="int4_gemm_kernel", graph=True)
 
 
-def wl_gemv_f16(torch, xmk, m=1, n=16384, k=4096, copies=4):
+def wl_gemv_f16(torch, xmk, m=1, n=16384, k=4096, copies=4, rhs_t=False):
     """Dense fp16 small-row GEMM, the shape class the reference's own tile table is mostly made of
     (`1_16384_4096`, xla/service/gpu/xetla/gemm/gemm.cc:33): weight-bandwidth bound, so reported as
     HBM GB/s.  K-split through xmk_gemm_ws with caller scratch when the planner asks for one.  The
     launches rotate through `copies` weight sets (4 x 134 MB > the 256 MB last-level cache)."""
     G = gen(torch)
     a = G.normal((m, k), 601, dtype=torch.float16)
-    bs = [G.normal((k, n), 602 + c, k ** -0.5, dtype=torch.float16) for c in range(copies)]
+    bs = [G.normal((n, k) if rhs_t else (k, n), 602 + c, k ** -0.5, dtype=torch.float16) for c in range(copies)]
     out = torch.empty((m, n), dtype=torch.float16, device="cuda")
-    need = xmk.gemm_workspace_bytes(a, bs[0], out)
+    need = xmk.gemm_workspace_bytes(a, bs[0], out, rhs_transpose=rhs_t)
     ws = torch.empty((max(need, 16),), dtype=torch.uint8, device="cuda") if need else None
     state = [0]
 
     def fn():
         b = bs[state[0] % copies]
         state[0] += 1
-        xmk.run_gemm(a, b, out, workspace=ws)
-    return dict(name=f"gemm_f16_m{m}_n{n}_k{k}", fn=fn, flops=2.0 * m * n * k, bytes=2.0 * (m * k + k * n + m * n),
+        xmk.run_gemm(a, b, out, rhs_transpose=rhs_t, workspace=ws)
+    return dict(name=f"gemm_f16_m{m}_n{n}_k{k}{'_rhsT' if rhs_t else ''}", fn=fn, flops=2.0 * m * n * k, bytes=2.0 * (m * k + k * n + m * n),
                 bound="hbm", dtype="f16", graph=True,
-                kernel=xmk.gemm_policy_name(m, n, k, False, xmk.F16, xmk.F16) + (" + splitk_reduce_kernel" if need else ""),
+                kernel=xmk.gemm_policy_name(m, n, k, rhs_t, xmk.F16, xmk.F16) + (" + splitk_reduce_kernel" if need else ""),
                 note=f"xmk_gemm_ws, {need} bytes of K-split scratch" if need else "xmk_gemm, unsplit")
 
 
@@ -463,6 +463,7 @@ WORKLOADS = {
     "gemm_c1": lambda t, x: wl_gemm(t, x, 512, 4096, 4096, bias=True),
     "lib_gemm_8192": lambda t, x: wl_lib_gemm(t, x),
     "gemv_f16_m1": lambda t, x: wl_gemv_f16(t, x, 1),
+    "gemv_f16_m1_rhsT": lambda t, x: wl_gemv_f16(t, x, 1, rhs_t=True),
     "gemv_f16_m4_vocab": lambda t, x: wl_gemv_f16(t, x, 4, 50400, 4096, copies=2),
     "int4_m1": lambda t, x: wl_int4(t, x, 1),
     "int4_m8": lambda t, x: wl_int4(t, x, 8),
@@ -471,7 +472,7 @@ WORKLOADS = {
     "fp8_8192_kn": lambda t, x: wl_fp8(t, x, 8192, 8192, 8192, rhs_t=False),
     "gptj_decode": lambda t, x: wl_gptj_decode(t, x),
 }
-ALSO = ["fmha", "fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "lib_gemm_8192", "gemm_c1", "gemv_f16_m1", "gemv_f16_m4_vocab", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "fp8_8192_kn", "gptj_decode"]
+ALSO = ["fmha", "fmha_bwd_causal", "gemm_8192", "gemm_8192_rhsT", "lib_gemm_8192", "gemm_c1", "gemv_f16_m1", "gemv_f16_m1_rhsT", "gemv_f16_m4_vocab", "int4_m1", "int4_m8", "int4_m32", "fp8_8192", "fp8_8192_kn", "gptj_decode"]
 
 
 def measure(torch, xmk, key, steps, warmup):

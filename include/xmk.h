@@ -137,9 +137,9 @@ int xmk_gemm_qkv(const xmk_gemm_desc* desc, void* out_k, void* out_v, void* stre
 /* Name of the tile policy xmk_gemm would pick for (m, n, k): the counterpart
  * of selectXetlaGemmConfig (xetla/gemm/gemm.cc:286-308).  Returns a static
  * string: "mfma_<BM>x<BN>x<BK>_..." for a matrix-core tile,
- * "stream_rows_8x512_w8" for the streaming kernel that one to eight rows
- * against a very wide [k,n]-stored matrix take (packed, aligned operands
- * assumed). */
+ * "stream_rows_8x512_w8" for the streaming kernels that a few rows against
+ * a wide matrix take, in either storage order of B (packed, aligned
+ * operands assumed). */
 const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int32_t rhs_transpose,
                                  int32_t dtype_in, int32_t dtype_out);
 

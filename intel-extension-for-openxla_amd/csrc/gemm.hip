@@ -199,8 +199,12 @@ extern "C" const char* xmk_gemm_policy_name(int64_t m, int64_t n, int64_t k, int
   if (dtype_in == XMK_S8 && dtype_out == XMK_S32) return "mfma_s8_128x128x64";
   if (!sixteen || !(dtype_out == dtype_in || dtype_out == XMK_F32)) return "generic_64x64";
   // (packed, aligned operands assumed, as everywhere in this query)
-  const bool rows_ok = !rhs_transpose && m >= 1 && m <= kRowsMaxM && n % 8 == 0 && k % 8 == 0;
-  return kPolicies[select_policy(m, n, k, 1, rows_ok)].name;
+  int rows_kind = kRowsNone;
+  if (m >= 1 && m <= kRowsMaxM && k % 8 == 0) {
+    if (!rhs_transpose && n % 8 == 0) rows_kind = kRowsMC;
+    if (rhs_transpose && k <= kColsMaxK) rows_kind = kRowsKC;
+  }
+  return kPolicies[select_policy(m, n, k, 1, rows_kind, !rhs_transpose)].name;
 }
 
 namespace {
@@ -215,16 +219,15 @@ bool direct_ok(const xmk_matrix& lhs, const xmk_matrix& rhs) {
          lhs.num_cols % 8 == 0 && rhs.num_cols % 8 == 0;
 }
 
-// Whether the streaming kernel for a few rows (gemm_rows.hip) can run this descriptor's product.
-bool rows_ok_desc(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k) {
-  if (d->out.transpose || d->lhs.transpose || d->rhs.transpose || !direct_ok(d->lhs, d->rhs) ||
-      !xmk::aligned(d->out.data, 16))
-    return false;
-  if (d->dtype_in != XMK_BF16 && d->dtype_in != XMK_F16) return false;
+// Which streaming kernel for a few rows (gemm_rows.hip) can run this descriptor's product, if any.
+int rows_kind_desc(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k) {
+  if (d->out.transpose || d->lhs.transpose || !direct_ok(d->lhs, d->rhs) || !xmk::aligned(d->out.data, 16))
+    return kRowsNone;
+  if (d->dtype_in != XMK_BF16 && d->dtype_in != XMK_F16) return kRowsNone;
   GemmParams p{};
   p.M = (int)m; p.N = (int)n; p.K = (int)k;
   p.lda = d->lhs.leading_dim_stride; p.ldb = d->rhs.leading_dim_stride;
-  return gemm_rows_applicable(p, false, true);
+  return gemm_rows_applicable(p, false, d->rhs.transpose == 0);
 }
 
 // K slices worth using for a plain 16-bit GEMM of this shape when scratch is available: few
@@ -239,24 +242,26 @@ int plan_splitk(const xmk_gemm_desc* d, int64_t m, int64_t n, int64_t k, int* po
   const char* forced_env = getenv("XMK_GEMM_SPLITK");
   const int forced = forced_env ? atoi(forced_env) : 0;
   if (forced >= 1) return divides(forced) ? forced : 1;
-  const bool rows_ok = rows_ok_desc(d, m, n, k) && (forced_policy() < 0 || forced_policy() == kRowsPolicy);
-  if (const TunedShape* t = tuned_shape(m, n, k); forced_policy() < 0 && t && t->ksplit >= 1 && divides(t->ksplit) &&
+  const int rows_kind = (forced_policy() < 0 || forced_policy() == kRowsPolicy) ? rows_kind_desc(d, m, n, k) : kRowsNone;
+  const bool rows_ok = rows_kind != kRowsNone;
+  // (the table was measured with B stored [K, N])
+  if (const TunedShape* t = tuned_shape(m, n, k); forced_policy() < 0 && !d->rhs.transpose && t && t->ksplit >= 1 && divides(t->ksplit) &&
                                                   (t->policy != kRowsPolicy || rows_ok)) {
     if (t->ksplit > 1) *policy = t->policy;
     return t->ksplit;
   }
-  if (rows_ok && xmk::ceil_div(n, (int64_t)kRowsDefaultBN) >= kRowsEnoughBlocks) return 1;  // streamed in one launch
+  if (rows_streams_by_default(rows_kind, m, n)) return 1;  // streamed in one launch
   if (rows_ok && forced_policy() == kRowsPolicy) {
     // The streaming kernel forced on a narrower matrix (tests, the autotuner): slices until its narrowest
     // column blocks are about one work-group per CU, each slice keeping 512 rows (a batch of 64 per wave).
-    const int64_t blocks = xmk::ceil_div(n, (int64_t)kRowsMinBN);
+    const int64_t blocks = xmk::ceil_div(n, (int64_t)(rows_kind == kRowsMC ? kRowsMinBN : kColsBN));
     int ks = 1;
     if (blocks < kRowsEnoughBlocks)
       while (ks < 16 && blocks * ks < 256 && k % (ks * 2 * 8) == 0 && k / (ks * 2) >= 512) ks *= 2;
     if (ks > 1) *policy = kRowsPolicy;
     return ks;
   }
-  const Policy& pol = kPolicies[select_policy(m, n, k)];
+  const Policy& pol = kPolicies[select_policy(m, n, k, 1, kRowsNone, !d->rhs.transpose)];
   const int64_t tiles = xmk::ceil_div(m, pol.bm) * xmk::ceil_div(n, pol.bn);
   int ks = 1;
   while (ks < 8 && tiles * ks * 2 <= 256 && k % (ks * 2 * 8) == 0 && k / (ks * 2) >= 512) ks *= 2;
@@ -450,10 +455,11 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int p
     const bool a_mc = lhs.transpose != 0;   // stored [K, M]
     const bool b_mc = rhs.transpose == 0;   // stored [K, N]
     const int batch = qkv ? 3 : (int)d->batch_size;
-    const bool rows_ok = fast && gemm_rows_applicable(p, a_mc, b_mc);
+    const int rows_kind = fast ? gemm_rows_applicable(p, a_mc, b_mc) : kRowsNone;
     // the forced policy first, then the K-split planner's, then the table and the rules
-    const int pol = (forced_policy() < 0 && policy >= 0 && policy < kNumPolicies && (policy != kRowsPolicy || rows_ok))
-                        ? policy : select_policy(m, n, k, batch, rows_ok);
+    const int pol = (forced_policy() < 0 && policy >= 0 && policy < kNumPolicies &&
+                     (policy != kRowsPolicy || rows_kind != kRowsNone))
+                        ? policy : select_policy(m, n, k, batch, rows_kind, b_mc);
     xmk::trace("gemm m=%lld n=%lld k=%lld batch=%lld lhs_t=%d rhs_t=%d epilogue=%d beta=%g -> %s",
                (long long)m, (long long)n, (long long)k, (long long)d->batch_size, lhs.transpose,
                rhs.transpose, d->epilogue, d->beta, gather ? kGatherPolicy.name : kPolicies[pol].name);
@@ -468,7 +474,7 @@ int run_gemm(const xmk_gemm_desc* d, void* out1, void* out2, void* stream, int p
       return xmk::check_launch("gemm");
     }
     if (pol == kRowsPolicy) {
-      launch_gemm_rows(p, din == XMK_BF16, dout == XMK_F32, batch, st);
+      launch_gemm_rows(p, b_mc, din == XMK_BF16, dout == XMK_F32, batch, st);
       return xmk::check_launch("gemm");
     }
     if (din == XMK_BF16) {

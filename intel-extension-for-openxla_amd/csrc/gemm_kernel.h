@@ -668,6 +668,12 @@ constexpr int kRowsEnoughBlocks = 192;  // work-groups from which on a launch pu
 // m = 1: 27.7 / 28.5, m = 4: 27.4 / 31.1; n = 12288, m = 8: 25.9 / 32.2; n = 4096, k = 16384, m = 4:
 // 30.1 / 36.8: below that width a launch is over before the stream has paid for its start and end.
 constexpr int kRowsDefaultBN = 128;
+// B stored [N, K] streams in blocks of 64 output columns and is the default for up to four rows from 12288
+// columns on (fp16, k = 4096, microseconds, matrix-core kernel against streaming: n = 50400, m = 1: 89.2 /
+// 78.6, m = 4: 90.1 / 80.8, m = 8: 91.4 / 95.6; n = 32000, m = 4: 61.6 / 49.5; n = 16384, m = 4: 33.6 / 25.5).
+constexpr int kColsBN = 64;
+constexpr int kColsMaxK = 16384;  // reduction length its register-resident pieces of A allow
+enum : int { kRowsNone = 0, kRowsMC = 1, kRowsKC = 2 };  // which streaming kernel the operands allow
 
 // Tile choice, the role of selectXetlaGemmConfig (xetla/gemm/gemm.cc:286-308).  Shapes listed in the tuned table
 // (gemm_policy_table.h, written by autotune_gemm.py from measurements) take the policy
@@ -684,6 +690,10 @@ inline const TunedShape* tuned_shape(int64_t m, int64_t n, int64_t k) {
     if (t.m == m && t.n == n && t.k == k) return &t;
   return nullptr;
 }
+inline bool rows_streams_by_default(int rows_kind, int64_t m, int64_t n) {
+  return (rows_kind == kRowsMC && xmk::ceil_div(n, (int64_t)kRowsDefaultBN) >= kRowsEnoughBlocks) ||
+         (rows_kind == kRowsKC && m <= 4 && xmk::ceil_div(n, (int64_t)kColsBN) >= kRowsEnoughBlocks);
+}
 // XMK_GEMM_POLICY=<index>, or -1.  Read at every call (a getenv costs far less than a launch), so that the
 // autotuner can walk the policies inside one process.
 inline int forced_policy() {
@@ -693,14 +703,17 @@ inline int forced_policy() {
   }
   return -1;
 }
-// rows_ok: the operands meet the streaming kernel's conditions (gemm_rows_applicable); it is never chosen otherwise.
-inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1, bool rows_ok = false) {
+// rows_kind: which streaming kernel the operands allow (gemm_rows_applicable); it is never chosen otherwise.
+// tuned_ok: the operands have the layout the tuned table was measured with (B stored [K, N]).
+inline int select_policy(int64_t m, int64_t n, int64_t k, int64_t batch = 1, int rows_kind = kRowsNone,
+                         bool tuned_ok = true) {
+  const bool rows_ok = rows_kind != kRowsNone;
   auto usable = [&](int v) { return v >= 0 && v < kNumPolicies && (v != kRowsPolicy || rows_ok); };
   if (const int v = forced_policy(); usable(v)) return v;
-  if (batch == 1)
+  if (batch == 1 && tuned_ok)
     if (const TunedShape* t = tuned_shape(m, n, k); t && t->ksplit <= 1 && usable(t->policy)) return t->policy;
   // A few rows against a very wide matrix: stream it.
-  if (rows_ok && batch == 1 && xmk::ceil_div(n, kRowsDefaultBN) >= kRowsEnoughBlocks) return kRowsPolicy;
+  if (batch == 1 && rows_streams_by_default(rows_kind, m, n)) return kRowsPolicy;
   // Heuristic: the policy with the best estimated throughput = (what the tile sustains when the
   // device is full) x (share of the 256 CUs busy over the tile waves) x (share of the tiles' area
   // inside the matrix).  The per-tile figures are measured large-shape rates relative to 256x256.

@@ -287,9 +287,9 @@ def test_vocabulary_projection_n50400(xmk, oracle, m, rhs_t):
     path), fp16 like the reference's decode."""
     n, k = 50400, 4096
     dt, kind = oracle.F16, "f16"
-    # one to eight rows against [K, N] storage stream the matrix; the others take a matrix-core tile
+    # one to eight rows stream the matrix (either storage order); the others take a matrix-core tile
     streamed = xmk.gemm_policy_name(m, n, k, rhs_t, xmk.F16, xmk.F16) == "stream_rows_8x512_w8"
-    assert streamed == (m <= 8 and not rhs_t)
+    assert streamed == (m <= 8)
     a = oracle.from_f32(oracle.normal((m, k), 84, k ** -0.5), dt)
     b = oracle.from_f32(oracle.normal((n, k) if rhs_t else (k, n), 85, 1.0), dt)
     bias = oracle.from_f32(oracle.normal((n,), 86, 0.5), dt)
@@ -313,41 +313,47 @@ def test_vocabulary_projection_n50400(xmk, oracle, m, rhs_t):
     (5, 8, 264, "EPI_BIAS_RELU", 0.0),      # one lane's worth of columns
     (2, 33000, 512, "EPI_GELU", 0.0),       # enough column blocks to be chosen without being forced
     (7, 2048, 1000, "EPI_DEFAULT", 0.0),
+    (6, 1088, 5000, "EPI_BIAS", 0.0),       # [N, K] storage: two loads per row and wave, the second partly past K
 ])
 @pytest.mark.parametrize("with_ws", [False, True])
-def test_streamed_rows(xmk, oracle, monkeypatch, dt_name, m, n, k, epi, beta, with_ws):
-    """One to eight rows against a [K, N] matrix on the streaming kernel (policy 5; forced here, since the
-    smaller shapes would take a matrix-core tile), unsplit and K-split into caller scratch."""
+@pytest.mark.parametrize("rhs_t", [False, True])
+def test_streamed_rows(xmk, oracle, monkeypatch, dt_name, m, n, k, epi, beta, with_ws, rhs_t):
+    """One to eight rows against a [K, N] or an [N, K] matrix on the streaming kernels (policy 5; forced here,
+    since the smaller shapes would take a matrix-core tile), unsplit and K-split into caller scratch."""
     monkeypatch.setenv("XMK_GEMM_POLICY", "5")
     dt = getattr(oracle, dt_name)
     kind = _kind(dt, oracle)
     a = oracle.from_f32(oracle.normal((m, k), 90, k ** -0.5), dt)
-    b = oracle.from_f32(oracle.normal((k, n), 91, 1.0), dt)
+    b = oracle.from_f32(oracle.normal((n, k) if rhs_t else (k, n), 91, 1.0), dt)
     c = oracle.from_f32(oracle.normal((m, n), 92, 1.0), dt)
     bias = oracle.from_f32(oracle.normal((n,), 93, 0.5), dt) if "BIAS" in epi else None
-    _, ref = oracle.gemm(a, b, dt, dt, c=c, bias=bias, beta=beta, epilogue=getattr(oracle, epi))
-    assert xmk.gemm_policy_name(m, n, k, False, getattr(xmk, dt_name), getattr(xmk, dt_name)) == "stream_rows_8x512_w8"
+    _, ref = oracle.gemm(a, b, dt, dt, rhs_t=rhs_t, c=c, bias=bias, beta=beta, epilogue=getattr(oracle, epi))
+    assert xmk.gemm_policy_name(m, n, k, rhs_t, getattr(xmk, dt_name), getattr(xmk, dt_name)) == "stream_rows_8x512_w8"
     da, db, dc = to_dev(a, kind), to_dev(b, kind), to_dev(c, kind)
     ws = None
     if with_ws:
-        nbytes = xmk.gemm_workspace_bytes(da, db, dc)
+        nbytes = xmk.gemm_workspace_bytes(da, db, dc, rhs_transpose=rhs_t)
         ws = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device="cuda")
-    xmk.run_gemm(da, db, dc, c=dc, beta=beta, bias=None if bias is None else to_dev(bias, kind),
+    xmk.run_gemm(da, db, dc, rhs_transpose=rhs_t, c=dc, beta=beta, bias=None if bias is None else to_dev(bias, kind),
                  epilogue=getattr(xmk, epi), workspace=ws)
     torch.cuda.synchronize()
     _check(oracle, dc.float().cpu().numpy(), ref[0])
 
 
-def test_streamed_rows_batched_f32_out(xmk, oracle, monkeypatch):
-    """The streaming kernel with a batch, fp32 output and padded leading dimensions."""
+@pytest.mark.parametrize("rhs_t", [False, True])
+def test_streamed_rows_batched_f32_out(xmk, oracle, monkeypatch, rhs_t):
+    """The streaming kernels with a batch, fp32 output and padded leading dimensions."""
     monkeypatch.setenv("XMK_GEMM_POLICY", "5")
-    bsz, m, n, k, lda, ldb, ldc = 3, 4, 1000, 136, 144, 1008, 1004
+    bsz, m, n, k, lda, ldc = 3, 4, 1000, 136, 144, 1004
+    ldb = 152 if rhs_t else 1008  # stored [n, k] or [k, n]
+    brows = n if rhs_t else k
     dt, kind = oracle.BF16, "bf16"
     a = oracle.from_f32(oracle.normal((bsz, m, lda), 94, k ** -0.5), dt)
-    b = oracle.from_f32(oracle.normal((bsz, k, ldb), 95, 1.0), dt)
+    b = oracle.from_f32(oracle.normal((bsz, brows, ldb), 95, 1.0), dt)
     da, db = to_dev(a, kind), to_dev(b, kind)
     out = torch.full((bsz, m, ldc), -7.0, dtype=torch.float32, device="cuda")
-    d = xmk.GemmDesc(xmk.Matrix(da.data_ptr(), 0, m, k, m * lda, lda), xmk.Matrix(db.data_ptr(), 0, k, n, k * ldb, ldb),
+    rhs = xmk.Matrix(db.data_ptr(), 1, n, k, n * ldb, ldb) if rhs_t else xmk.Matrix(db.data_ptr(), 0, k, n, k * ldb, ldb)
+    d = xmk.GemmDesc(xmk.Matrix(da.data_ptr(), 0, m, k, m * lda, lda), rhs,
                      xmk.Matrix(out.data_ptr(), 0, m, n, m * ldc, ldc), None, None, xmk.BF16, xmk.F32, bsz, 2.0, 0.0,
                      xmk.EPI_DEFAULT)
     xmk.run_gemm_desc(d)
@@ -355,7 +361,8 @@ def test_streamed_rows_batched_f32_out(xmk, oracle, monkeypatch):
     got = out.cpu().numpy()
     af, bf = oracle.to_f32(a, dt), oracle.to_f32(b, dt)
     for z in range(bsz):
-        ref = 2.0 * (af[z, :, :k].astype(np.float64) @ bf[z, :, :n].astype(np.float64))
+        bz = bf[z, :n, :k].T if rhs_t else bf[z, :k, :n]
+        ref = 2.0 * (af[z, :, :k].astype(np.float64) @ bz.astype(np.float64))
         _check(oracle, got[z, :, :n], ref.astype(np.float32))
     assert (got[:, :, n:] == -7.0).all(), "columns past N were written"
 
