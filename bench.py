@@ -31,6 +31,7 @@ TRAFFIC_BYTES = {
     "gemm_8192": (790500 * 2.0 + 131070) * 1024,
     "int4_m1": (17490 * 2.0 + 32) * 1024,
     "gemv_f16_m4_vocab": (203210 * 2.0 + 394) * 1024,
+    "gemv_f16_m1_rhsT": (65646 * 2.0 + 32) * 1024,
     "fp8_8192": (393620 * 2.0 + 131070) * 1024,
 }
 
