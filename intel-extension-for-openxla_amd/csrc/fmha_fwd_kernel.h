@@ -230,18 +230,30 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   const int vchunk = (lane % CPR) ^ vswz(lrow);
   const uint32_t voff = vchunk * 8 < H ? (uint32_t)((lrow * H + vchunk * 8) * 2) : kOob;
   const uint32_t lstride = (uint32_t)(LROWS * H * 2);  // global bytes between a wave's loads
-  // Half tile hh (32 rows from row 32 hh of K or V) into `stage`.  The per-load scalar offset is not
-  // range-checked by the hardware, so unless the half tile is known to be whole (FULL) rows past T
-  // are turned into out-of-range lane offsets, which load zeros.
-  auto issue_half = [&](auto FULL, const T* base, int hh, char* __restrict__ stage, const uint32_t* offs, int noffs) {
+  // Half tile hh (32 rows from row 32 hh of K or V) into `stage`.  Rows past T load zeros, in two ways.
+  // RANGED: every load gets a buffer descriptor of its own that ends with the last row (a handful of
+  // scalar instructions; a half tile wholly past T then touches no memory at all), so that the plain
+  // steps can run up to the end of the keys.  Otherwise one descriptor per half tile, the loads apart by
+  // a scalar offset, which the hardware does not range-check: rows past T become out-of-range lane offsets.
+  auto issue_half = [&](auto RANGED, const T* base, int hh, char* __restrict__ stage, const uint32_t* offs, int noffs) {
     const int rows_left = Tk - 32 * hh;  // may be <= 0 for the second half of the last tile
-    const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)(32 * hh) * H, 0x7fffffffu);
-    const bool full = decltype(FULL)::value || rows_left >= 32;
+    if constexpr (decltype(RANGED)::value) {
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const uint32_t off = (full || lrow + i * LROWS < rows_left) ? offs[i % noffs] : kOob;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(stage + (i * NW + wave) * 1024), 16, off,
-                                               i * lstride, 0, 0);
+      for (int i = 0; i < NL; ++i) {
+        const int rl = max(rows_left - i * LROWS, 0);
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)(32 * hh + i * LROWS) * H, (uint32_t)rl * (uint32_t)(H * 2));
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(stage + (i * NW + wave) * 1024), 16, offs[i % noffs], 0,
+                                                 0, 0);
+      }
+    } else {
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)(32 * hh) * H, 0x7fffffffu);
+      const bool full = rows_left >= 32;
+#pragma unroll
+      for (int i = 0; i < NL; ++i) {
+        const uint32_t off = (full || lrow + i * LROWS < rows_left) ? offs[i % noffs] : kOob;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(stage + (i * NW + wave) * 1024), 16, off,
+                                                 i * lstride, 0, 0);
+      }
     }
   };
 
@@ -453,11 +465,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   //     before that of half tile h;
   //   - waits until the loads that the NEXT step reads have landed (those sent two steps ago: the
   //     loads of this and the last step may stay in flight) and meets the other waves.
-  // MASKED steps: S_{h+1} touches the causal diagonal or the end of the keys; they also check every
-  // load against the end of K / V and wait for all loads (counting the loads that the last steps still send,
-  // and waiting only for the older ones, was measured: no gain), and a wave leaves out the work past its
-  // last half tile (nh).  PV / SC: whether there is a P V product (not in step 0) and an S product
-  // (not in the last step) to run.
+  // MASKED steps: S_{h+1} may touch the causal diagonal or the end of the keys: the mask is applied where a
+  // wave needs one, and a wave leaves out the work past its last half tile (nh).  Loads and waits are those
+  // of the plain form: ranged loads, which may reach past the keys, and a counted wait.  A masked step
+  // takes 1.1-1.4 us where a plain one takes 0.86 (per-wave timestamps, [8,32,2048,128]), mask or no
+  // mask, so the plain form runs wherever no wave needs a mask.  PV / SC: whether there is a P V product
+  // (not in step 0) and an S product (not in the last step) to run.
   float mref_c, alpha_c = 1.0f;  // exponent reference of S_h; factor O has to be multiplied by before P V of h
   bool moved_c = false;          // whether alpha_c differs from 1 for some row
   auto step = [&](auto MASKED, auto PV, auto SC, auto HSC, int h) {
@@ -503,8 +516,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
     // cycles, under which the reads' latency passes.
     if (active) static_for<D>(fetch);
     __builtin_amdgcn_sched_barrier(0);
-    if (!masked || h + 4 < nhalf) issue_half(std::integral_constant<bool, !masked>{}, K, h + 4, kfree, koff, KV);
-    if (!masked || h + 2 < nhalf) issue_half(std::integral_constant<bool, !masked>{}, V, h + 2, vfree, &voff, 1);
+    if constexpr (sco) {  // (the last step has nothing left to send)
+      issue_half(true_type{}, K, h + 4, kfree, koff, KV);
+      issue_half(true_type{}, V, h + 2, vfree, &voff, 1);
+    }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr ((HS & 1) == 1 && sco) take_bias((h + 1) / 2);
     if (active) {
@@ -589,7 +604,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
       moved_c = moved_n;
     }
     }(kst0 + ((HS + 1) % NST) * HALF, vst0 + ((HS + 3) % NST) * HALF, kst0 + HS * HALF, vst0 + ((HS + 2) % NST) * HALF);
-    if constexpr (masked || BIAS == 2) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+    // The loads of this step and of the one before may stay in flight; the last step sends none and ends
+    // with all of them landed, since the output rows are staged where K and V were.
+    if constexpr (!sco || BIAS == 2) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
     else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(4 * NL));
     __builtin_amdgcn_s_barrier();
   };
@@ -603,11 +620,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   issue_half(false_type{}, K, 0, kst0, koff, KV);
   issue_half(false_type{}, K, 1, kst0 + HALF, koff, KV);
   issue_half(false_type{}, V, 0, vst0, &voff, 1);
-  if (nhalf > 2) issue_half(false_type{}, K, 2, kst0 + 2 * HALF, koff, KV);
-  if (nhalf > 2) issue_half(false_type{}, K, 3, kst0 + 3 * HALF, koff, KV);
+  issue_half(true_type{}, K, 2, kst0 + 2 * HALF, koff, KV);  // (ranged: past the keys they touch no memory, and
+  issue_half(true_type{}, K, 3, kst0 + 3 * HALF, koff, KV);  //  the count of loads in flight is the same for every T)
   issue_half(false_type{}, V, 1, vst0 + HALF, &voff, 1);
-  if (nhalf > 2) __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(4 * NL));
-  else __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(2 * NL));
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(4 * NL));
   __builtin_amdgcn_s_barrier();
   take_bias(0);
   scores(kst0, sa);
@@ -622,24 +638,40 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   __builtin_amdgcn_s_barrier();
   step(true_type{}, false_type{}, true_type{}, hs0{}, 0);
 
-  // Steps 1 .. nhalf-1, four to a trip.  A step is masked when the half tile after its own touches the
-  // causal diagonal or the end of the keys; the steps of the two last tiles (three when the last is
-  // ragged) always take the masked form, so that the plain form always has whole half tiles to load.
-  const int last_plain = (Tk % BC != 0) ? nblk - 3 : nblk - 2;  // plain steps load whole half tiles, unchecked
-  const int first_masked = CAUSAL ? min(q0 / BC, last_plain) : last_plain;
-  int j = 1;
-  for (; j + 1 < first_masked; j += 2) {
-    step(false_type{}, true_type{}, true_type{}, hs1{}, 2 * j - 1);
-    step(false_type{}, true_type{}, true_type{}, hs2{}, 2 * j);
-    step(false_type{}, true_type{}, true_type{}, hs3{}, 2 * j + 1);
-    step(false_type{}, true_type{}, true_type{}, hs0{}, 2 * j + 2);
+  // Steps 1 .. nhalf-2.  A step's S product is that of half tile h + 1: it needs the masked form from the
+  // first half tile on that touches the causal diagonal of the work-group's first row or holds keys past T;
+  // before that every wave has all of its rows below the keys and the plain form (whose loads are ranged)
+  // runs.  Plain steps go four to a trip (stage positions 1, 2, 3, 0); the causal diagonal starts in the
+  // middle of such a group, hence the two extra plain steps and the two masked ones that follow them,
+  // after which the masked steps go on from stage position 1 like the plain ones.  (One loop that picks a
+  // step's copy by h % 4 was tried: it spilled registers in the step and ran at a third of the rate.)
+  const int hmask = min(CAUSAL ? q0 / 32 : 0x7fffffff, Tk / 32);  // first half tile that needs a mask
+  const int hend = nhalf - 1;                                     // the last step, which has no S product
+  const int hplain = min(hend, hmask - 1);                        // steps below it may be plain
+  int h = 1;
+  for (; h + 3 < hplain; h += 4) {
+    step(false_type{}, true_type{}, true_type{}, hs1{}, h);
+    step(false_type{}, true_type{}, true_type{}, hs2{}, h + 1);
+    step(false_type{}, true_type{}, true_type{}, hs3{}, h + 2);
+    step(false_type{}, true_type{}, true_type{}, hs0{}, h + 3);
   }
-  for (; j < nblk; j += 2) {
-    step(true_type{}, true_type{}, true_type{}, hs1{}, 2 * j - 1);
-    step(true_type{}, true_type{}, true_type{}, hs2{}, 2 * j);
-    if (j + 1 < nblk) {
-      step(true_type{}, true_type{}, true_type{}, hs3{}, 2 * j + 1);
-      step(true_type{}, true_type{}, true_type{}, hs0{}, 2 * j + 2);
+  if (h + 1 < hplain) {
+    step(false_type{}, true_type{}, true_type{}, hs1{}, h);
+    step(false_type{}, true_type{}, true_type{}, hs2{}, h + 1);
+    h += 2;
+    if (h < hend) {  // (hend is odd, h is 3 mod 4: a further step is followed by another)
+      step(true_type{}, true_type{}, true_type{}, hs3{}, h);
+      step(true_type{}, true_type{}, true_type{}, hs0{}, h + 1);
+      h += 2;
+    }
+  }
+  for (; h < hend; h += 2) {
+    step(true_type{}, true_type{}, true_type{}, hs1{}, h);
+    step(true_type{}, true_type{}, true_type{}, hs2{}, h + 1);
+    if (h + 2 < hend) {
+      step(true_type{}, true_type{}, true_type{}, hs3{}, h + 2);
+      step(true_type{}, true_type{}, true_type{}, hs0{}, h + 3);
+      h += 2;
     }
   }
   // The last step (half tile nhalf-1, odd: no further S) and the P V product of that half tile.
