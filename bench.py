@@ -27,7 +27,7 @@ RAMP_SECONDS = 0.25                                      # untimed launches befo
 # kernels (profiles/hbm_traffic_pmc.txt says which build and when), not of the run that prints them: they are
 # to be measured again whenever one of these kernels changes.  A workload without a measurement reports null.
 TRAFFIC_BYTES = {
-    "fmha_causal": (221210 * 2.0 + 131070) * 1024,
+    "fmha_causal": (204930 * 2.0 + 131070) * 1024,
     "gemm_8192": (790500 * 2.0 + 131070) * 1024,
     "int4_m1": (17490 * 2.0 + 32) * 1024,
     "gemv_f16_m4_vocab": (203210 * 2.0 + 394) * 1024,
