@@ -69,8 +69,18 @@ __device__ __forceinline__ half8 permute_act(u32x4 d, uint32_t sel_lo, uint32_t 
 }
 
 constexpr uint32_t kOob = 0x80000000u;
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+// s_waitcnt immediate: at most n vector-memory loads outstanding, the other counters not waited for.
+constexpr int vmcnt_imm(int n) { return (n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8); }
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// 16 bytes per lane from byte offset voff + soff of a buffer straight into LDS: lane l's land at lds + 16 l
+// (zeros where the offset is out of range).  (A function of its own: written into a kernel's body, the
+// builtin makes the host pass drop the kernel's launch stub.)
+__device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t r, char* lds, uint32_t voff, uint32_t soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)lds, 16, voff, soff, 0, 0);
 }
 
 template <int NWORDS>
@@ -150,6 +160,13 @@ __device__ __forceinline__ void static_steps(F&& f) {
   }
 }
 
+// The first activation staging buffer of a work-group; the waves' partial sums take its place after the K loop.
+template <int STAGE_BYTES, int SUMS>
+union alignas(1024) StageOrSums {
+  char stage[STAGE_BYTES];
+  float sums[SUMS];
+};
+
 template <int W, int MT, int RI, int SPG, int NW, bool SK, bool SPREAD, int SDIV = 1>
 __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0, int mixed) {
   // mixed (two K-split products of equal width): the products alternate from one block to the next, and
@@ -172,7 +189,27 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   static_assert(!SPREAD || (MT == 1 && (RI == 1 || RI == 2)), "spread rows: one tile, one or two live elements per lane");
   constexpr int ROWS = SPREAD ? 4 * RI : (MT == 2 ? 32 : (RI == 4 ? 16 : RI));  // rows the block reduces
   constexpr int ESTEP = SPREAD ? 4 / RI : 1;  // live accumulator elements are 0, ESTEP, ...
-  __shared__ float red[NW][ROWS][NCOL];
+  // kExact: work-groups that own their whole reduction, of eight waves, or four with several rows (see the
+  // fetch below).
+  // kStage: such work-groups with more than one row bring the activations in through LDS.  Read straight into
+  // the matrix instruction's operand layout (lane -> row l % 16, 16 bytes of it), a load touches 64 separate
+  // 64-byte pieces, one per lane group, because neighbouring lanes hold different rows: measured at 32 rows,
+  // the CU's load path spent 64 cycles on every such load against 16 for a load of the packed weights, 20
+  // thousand of the launch's 33 thousand cycles.  Instead each wave copies its group's ROWS x (64 SPG) bytes
+  // global -> LDS with lanes along the rows (16 per 1 KiB load), into a region of its own, and picks the
+  // operand fragments up with 16-byte LDS reads.  Chunk c of row r lives in slot c ^ sw(r) of the row, which
+  // spreads the 16 rows a read phase touches over all banks.  No barrier: a wave reads what it loaded itself,
+  // and the vector-memory counter orders the two.
+  constexpr bool kExact = (NW == 8 || (NW == 4 && ROWS > 1)) && !SK;
+  constexpr bool kStage = kExact && ROWS > 1 && !(SPG == 1 && SPREAD);  // (groups of 32, up to 8 rows: 4-5 % slower staged)
+  constexpr int CPR = 4 * SPG;                              // 16-byte chunks per activation row and group
+  constexpr int NI = kStage ? (ROWS * CPR + 63) / 64 : 0;   // 1 KiB loads per group and wave
+  constexpr int REGION = NI * 1024;                         // bytes per wave and buffer
+  // (the 256 bytes behind the waves' regions stay zero: the operand rows that carry no activation row read them)
+  constexpr int STAGE_BYTES = kStage ? NW * REGION + 256 : 16;
+  __shared__ StageOrSums<STAGE_BYTES, NW * ROWS * NCOL> s0;  // two objects, so that the compiler can tell a read
+  __shared__ alignas(1024) char s1[STAGE_BYTES];             // of one buffer from a load into the other
+  float (*red)[ROWS][NCOL] = reinterpret_cast<float (*)[ROWS][NCOL]>(s0.sums);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -184,11 +221,12 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
 
   // Buffer descriptors: hardware bounds checking zero-fills lanes that are out of range
   // (offset kOob), and the per-lane byte offsets below never change inside the K loop.
-  const __amdgpu_buffer_rsrc_t r_w = make_rsrc(qw, (uint32_t)((size_t)(K / 8) * N * 4));
-  const __amdgpu_buffer_rsrc_t r_s = make_rsrc(scales, (uint32_t)((size_t)(ngroups / SDIV) * N * 2));
-  const __amdgpu_buffer_rsrc_t r_z = make_rsrc(zeros, (uint32_t)((size_t)(ngroups / SDIV) * N * 2));
+  const __amdgpu_buffer_rsrc_t r_none = make_rsrc(qw, 0);
+  const __amdgpu_buffer_rsrc_t r_w_all = make_rsrc(qw, (uint32_t)((size_t)(K / 8) * N * 4));
+  const __amdgpu_buffer_rsrc_t r_s_all = make_rsrc(scales, (uint32_t)((size_t)(ngroups / SDIV) * N * 2));
+  const __amdgpu_buffer_rsrc_t r_z_all = make_rsrc(zeros, (uint32_t)((size_t)(ngroups / SDIV) * N * 2));
   // (the 32 rows of this launch only: the byte count must fit the descriptor's 32 bits for any M)
-  const __amdgpu_buffer_rsrc_t r_a = make_rsrc(act + (size_t)m_base * K, (uint32_t)((size_t)min(M - m_base, 32) * K * 2));
+  const __amdgpu_buffer_rsrc_t r_a_all = make_rsrc(act + (size_t)m_base * K, (uint32_t)((size_t)min(M - m_base, 32) * K * 2));
   const uint32_t voff_w = col_ok ? (uint32_t)((kg * N + n0) * 4) : kOob;
   const uint32_t voff_sz = col_ok ? (uint32_t)(n0 * 2) : kOob;
   uint32_t voff_a[MT];
@@ -197,6 +235,27 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     const int m = SPREAD ? col16 / ESTEP : mt * 16 + col16;
     const bool fed = !SPREAD || col16 % ESTEP == 0;  // MFMA rows ESTEP r carry activation row r, the others zeros
     voff_a[mt] = (fed && m_base + m < M) ? (uint32_t)((m * K + 8 * kg) * 2) : kOob;
+  }
+
+  uint32_t voff_st[kStage ? NI : 1];  // staging load i: this lane's chunk of the group's activations
+  uint32_t rd_off[SPG];               // k-step s: where this lane's operand fragment of tile 0 sits in the wave's region
+  if constexpr (kStage) {
+    constexpr int RPS = 16 / CPR;  // rows per 256 bytes of LDS
+    const int rows_here = min(M - m_base, ROWS);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int l = i * 64 + lane, row = l / CPR, chunk = (l % CPR) ^ ((row / RPS) % CPR);
+      voff_st[i] = row < rows_here ? (uint32_t)((row * K + chunk * 8) * 2) : kOob;
+    }
+    const int lr = SPREAD ? col16 / ESTEP : col16;
+    const bool fed = !SPREAD || col16 % ESTEP == 0;
+    const uint32_t at = fed ? (uint32_t)(wave * REGION + (lr * CPR + (kg ^ ((lr / RPS) % CPR))) * 16) : (uint32_t)(NW * REGION);
+#pragma unroll
+    for (int s = 0; s < SPG; ++s) rd_off[s] = at ^ (uint32_t)(s << 6);
+    if (lane < 16) {
+      *reinterpret_cast<u32x4*>(s0.stage + NW * REGION + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(s1 + NW * REGION + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    }
   }
 
   floatx4 acc[MT][W];
@@ -222,31 +281,42 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     Words<(W + 1) / 2> sc, zp;
     u32x4 a[SPG][MT];
   };
-  // kExact (eight-wave work-groups that own their whole reduction): a fetch past the wave's last group is
-  // still issued, with every lane out of range (no memory access, zeros returned), and the groups run as
-  // straight-line code, so that the sequence of loads is the same on every path and the counted waits
-  // the compiler places before a group's arithmetic leave the next group's loads in flight.  The other
-  // shapes keep a loop with fetches behind branches, whose waits drain the prefetch at every turn: measured
-  // on one device, the exact form is 9-12 % faster at 8 rows and 5 % at 32 (k 4096, n 16384), 3-5 % slower on
-  // the sixteen-wave one-row kernel and 1.4 % slower over a decode step (four-wave and K-split launches).
-  constexpr bool kExact = NW == 8 && !SK;
-  auto fetch = [&](int g_asked, GroupData& d, bool live) {
+  // kExact (work-groups that own their whole reduction: eight waves, or four with more than one row): a fetch
+  // past the wave's last group is still issued, through descriptors of no bytes (no memory access, zeros
+  // returned), and the groups run as straight-line code, so that the sequence of loads is the same on every
+  // path and the counted waits the compiler places before a group's arithmetic leave the next group's loads
+  // in flight.  The other shapes keep a loop with fetches behind branches, whose waits drain the prefetch at
+  // every turn: measured on one device, the exact form is 9-12 % faster at 8 rows and 5 % at 32 (k 4096,
+  // n 16384), 3-5 % slower on the sixteen-wave one-row kernel, and level on the K-split launches; on the
+  // four-wave form it is 1.4 % slower over a decode step by itself and 1.5 % faster together with the staged
+  // activations.
+  auto fetch = [&](int g_asked, GroupData& d, bool live, auto which) {
     // (a fetch past the end uses group 0's scalar offsets, so that kOob plus the scalar offset cannot wrap
     //  around 32 bits whatever the unit that checks the range adds up)
     const int g = live ? g_asked : 0;
     // (wave-uniform; said explicitly, or the compiler wraps each of the two loads in a loop over lane values)
     const uint32_t so = __builtin_amdgcn_readfirstlane((uint32_t)((g / SDIV) * N * 2));
-    const uint32_t vsz = live ? voff_sz : kOob, vw = live ? voff_w : kOob;
+    // (a fetch past the end: descriptors of no bytes, four scalar selects instead of a vector select per load)
+    const __amdgpu_buffer_rsrc_t r_s = live ? r_s_all : r_none, r_z = live ? r_z_all : r_none;
+    const __amdgpu_buffer_rsrc_t r_a = live ? r_a_all : r_none, r_w = live ? r_w_all : r_none;
+    const uint32_t vsz = voff_sz, vw = voff_w;
     constexpr bool kPinned = kExact;
     if constexpr (kPinned) __builtin_amdgcn_sched_barrier(0);  // the loads stay together and in this order
     d.sc = load_halves<W>(r_s, vsz, so);
     d.zp = load_halves<W>(r_z, vsz, so);
+    if constexpr (kStage) {
+      char* dst = (which == 0 ? s0.stage : s1) + wave * REGION;
 #pragma unroll
-    for (int s = 0; s < SPG; ++s)
+      for (int i = 0; i < NI; ++i)
+        load_to_lds(r_a, dst + i * 1024, voff_st[i], (uint32_t)(g * SPG * 64));
+    } else {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        d.a[s][mt] = __builtin_bit_cast(
-            u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_a, live ? voff_a[mt] : kOob, (uint32_t)((g * SPG + s) * 64), 0));
+      for (int s = 0; s < SPG; ++s)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          d.a[s][mt] = __builtin_bit_cast(
+              u32x4, __builtin_amdgcn_raw_buffer_load_b128(r_a, voff_a[mt], (uint32_t)((g * SPG + s) * 64), 0));
+    }
 #pragma unroll
     for (int s = 0; s < SPG; ++s)
       d.w[s] = load_words<W>(r_w, vw, (uint32_t)((g * 4 * SPG + s * 4) * N * 4));
@@ -259,7 +329,7 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  auto compute = [&](const GroupData& cur) {
+  auto compute = [&](const GroupData& cur, auto which) {
     floatx4 d[MT][W], asum[MT], noff[MT];
     half8 a[SPG][MT];
     // (kExact: derived from the constant that the fetch has just laundered, see there)
@@ -276,7 +346,12 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     for (int s = 0; s < SPG; ++s)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        a[s][mt] = permute_act(cur.a[s][mt], sel_lo, sel_hi);
+        u32x4 raw;
+        if constexpr (kStage)
+          raw = *reinterpret_cast<const u32x4*>((which == 0 ? s0.stage : s1) + rd_off[s] + mt * (16 * CPR * 16));
+        else
+          raw = cur.a[s][mt];
+        a[s][mt] = permute_act(raw, sel_lo, sel_hi);
         noff[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[s][mt], noffs.h, noff[mt], 0, 0, 0);
       }
 #pragma unroll
@@ -323,36 +398,46 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
     const int mine = g < gend ? (gend - g + NW - 1) / NW : 0;
     constexpr int kStraight = DEPTH == 3 ? 9 : 8;
     static_steps<0, DEPTH - 1>([&](auto j) {
-      fetch(g + j * NW, buf[j], j < mine);
+      fetch(g + j * NW, buf[j], j < mine, j);
       return true;
     });
     static_steps<0, kStraight>([&](auto i) {
       if (i >= mine) return false;
-      fetch(g + (i + DEPTH - 1) * NW, buf[(i + DEPTH - 1) % DEPTH], i + DEPTH - 1 < mine);
-      compute(buf[i % DEPTH]);
+      fetch(g + (i + DEPTH - 1) * NW, buf[(i + DEPTH - 1) % DEPTH], i + DEPTH - 1 < mine,
+            std::integral_constant<int, (decltype(i)::value + DEPTH - 1) % DEPTH>{});
+      compute(buf[i % DEPTH], std::integral_constant<int, decltype(i)::value % DEPTH>{});
       return true;
     });
     // long reductions: the rest in a loop (buf[j] holds group kStraight + j; kStraight is a multiple of DEPTH)
     for (int i = kStraight; i < mine;) {
       static_steps<0, DEPTH>([&](auto j) {
         if (i >= mine) return false;
-        fetch(g + (i + DEPTH - 1) * NW, buf[(j + DEPTH - 1) % DEPTH], i + DEPTH - 1 < mine);
-        compute(buf[j]);
+        fetch(g + (i + DEPTH - 1) * NW, buf[(j + DEPTH - 1) % DEPTH], i + DEPTH - 1 < mine,
+              std::integral_constant<int, (decltype(j)::value + DEPTH - 1) % DEPTH>{});
+        compute(buf[j], j);
         ++i;
         return true;
       });
     }
   } else {
-    if (g < gend) fetch(g, buf[0], true);
+    constexpr std::integral_constant<int, 0> b0{};
+    constexpr std::integral_constant<int, 1> b1{};
+    if (g < gend) fetch(g, buf[0], true, b0);
     while (g < gend) {
-      if (g + NW < gend) fetch(g + NW, buf[1], true);
-      compute(buf[0]);
+      if (g + NW < gend) fetch(g + NW, buf[1], true, b1);
+      compute(buf[0], b0);
       g += NW;
       if (g >= gend) break;
-      if (g + NW < gend) fetch(g + NW, buf[0], true);
-      compute(buf[1]);
+      if (g + NW < gend) fetch(g + NW, buf[0], true, b0);
+      compute(buf[1], b1);
       g += NW;
     }
+  }
+  if constexpr (kStage) {
+    // The partial sums below reuse the staging memory: every load into it has landed (the fetches past the end
+    // write zeros there) and every wave has read its last group.
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    __syncthreads();
   }
 
   // Lane holds rows 4*kg+i (+16 mt) of columns col16*W+c.
