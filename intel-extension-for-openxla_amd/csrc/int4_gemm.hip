@@ -169,6 +169,13 @@ union alignas(1024) StageOrSums {
 
 template <int W, int MT, int RI, int SPG, int NW, bool SK, bool SPREAD, int SDIV = 1>
 __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4Problem p1, int blocks0, int mixed) {
+  // Every argument the K loop needs is asked for here, so that the scalar loads of the argument block go out
+  // together and the kernel starts after one round trip to it.  (Left to itself the compiler fetched them in
+  // two or three dependent rounds in some instantiations: 0.25 us on a launch of 9.)
+  if constexpr (NW != 16)  // (the sixteen-wave one-row form: 8.8 -> 9.15 us with it)
+    asm volatile("" : : "s"(p0.act), "s"(p1.act), "s"(p0.qw), "s"(p1.qw), "s"(p0.scales), "s"(p1.scales), "s"(p0.zeros),
+                 "s"(p1.zeros), "s"(p0.m_base), "s"(p1.m_base), "s"(p0.M), "s"(p1.M), "s"(p0.K), "s"(p1.K), "s"(p0.N),
+                 "s"(p1.N), "s"(blocks0), "s"(mixed));
   // mixed (two K-split products of equal width): the products alternate from one block to the next, and
   // the alternation flips between the first and the second half of the K slices, so that work-groups
   // which are half a grid apart -- the ones that end up sharing a CU -- belong to different products
@@ -207,6 +214,8 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   constexpr int REGION = NI * 1024;                         // bytes per wave and buffer
   // (the 256 bytes behind the waves' regions stay zero: the operand rows that carry no activation row read them)
   constexpr int STAGE_BYTES = kStage ? NW * REGION + 256 : 16;
+  constexpr int kLoadsPerFetch = 2 + NI + SPG;  // scales, zero points, staging loads, weights: one instruction each
+  static_assert(SPG + kLoadsPerFetch < 64, "the wait below counts up to 63 loads");
   __shared__ StageOrSums<STAGE_BYTES, NW * ROWS * NCOL> s0;  // two objects, so that the compiler can tell a read
   __shared__ alignas(1024) char s1[STAGE_BYTES];             // of one buffer from a load into the other
   float (*red)[ROWS][NCOL] = reinterpret_cast<float (*)[ROWS][NCOL]>(s0.sums);
@@ -340,6 +349,11 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
       asum[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
       noff[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
+    // The staged activations of this group have landed once at most the loads issued after them are
+    // outstanding: this group's weights and the whole next fetch (always issued in this form).  Said
+    // explicitly: inside the loop that follows the straight-line groups the compiler left this wait out
+    // before the reads of one of the two buffers.
+    if constexpr (kStage) __builtin_amdgcn_s_waitcnt(vmcnt_imm(SPG + kLoadsPerFetch));
     // -sum_k a_k offset_k of the whole group first: it is the start value of every column's
     // accumulator chain, so that the chains end at sum_k a_k q_k with the unpack offsets gone.
 #pragma unroll
@@ -441,33 +455,91 @@ __global__ __launch_bounds__(NW * 64) void int4_gemm_kernel(Int4Problem p0, Int4
   }
 
   // Lane holds rows 4*kg+i (+16 mt) of columns col16*W+c.
+  // Q: columns per thread of the reduction below.  Where single values would take four rounds or more (32 rows
+  // on eight waves, 16 on four: measured 1.9 us at 32 rows), a lane's four columns of a row go to LDS as one
+  // 16-byte store and a thread of the reduction owns such a quad: one round of 16-byte reads.  With fewer
+  // rounds the quads are slower (one row 8.8 -> 9.25 us, eight rows 9.0 -> 9.55, decode step +1.3 %).
+  constexpr int Q = (W == 4 && ROWS * NCOL >= 4 * NW * 64) ? 4 : 1;
+  auto put = [&](int row, int i, int mt) {
+    if constexpr (Q == 4) {
+      *reinterpret_cast<floatx4*>(&red[wave][row][col16 * 4]) = floatx4{acc[mt][0][i], acc[mt][1][i], acc[mt][2][i], acc[mt][3][i]};
+    } else {
+#pragma unroll
+      for (int c = 0; c < W; ++c) red[wave][row][col16 * W + c] = acc[mt][c][i];
+    }
+  };
   if constexpr (SPREAD) {
 #pragma unroll
-    for (int j = 0; j < RI; ++j)
-#pragma unroll
-      for (int c = 0; c < W; ++c) red[wave][kg * RI + j][col16 * W + c] = acc[0][c][j * ESTEP];
+    for (int j = 0; j < RI; ++j) put(kg * RI + j, j * ESTEP, 0);
   } else if (RI == 4 || kg == 0) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int i = 0; i < RI; ++i)
-#pragma unroll
-        for (int c = 0; c < W; ++c) red[wave][mt * 16 + (RI == 4 ? 4 * kg : 0) + i][col16 * W + c] = acc[mt][c][i];
+      for (int i = 0; i < RI; ++i) put(mt * 16 + (RI == 4 ? 4 * kg : 0) + i, i, mt);
   }
   __syncthreads();
 
+  // Thread e of the reduction owns Q consecutive columns of one row: sums over the waves in wave order.
   const int rows = min(ROWS, M - m_base);
+  auto wave_sums = [&](int row, int col, float (&sum)[Q]) {
+    if constexpr (Q == 4) {
+      floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < NW; ++w) v += *reinterpret_cast<const floatx4*>(&red[w][row][col]);
+      sum[0] = v[0]; sum[1] = v[1]; sum[2] = v[2]; sum[3] = v[3];
+    } else {
+      sum[0] = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) sum[0] += red[w][row][col];
+    }
+  };
   if constexpr (SK) {
     // This work-group's partial sums, fp32, no epilogue: the consumer adds the slices up.
     float* mine = partial + (size_t)blockIdx.y * 32 * N;
-    for (int e = threadIdx.x; e < rows * NCOL; e += NW * 64) {
-      const int row = e / NCOL, col = e % NCOL;
+    for (int e = threadIdx.x; e < rows * (NCOL / Q); e += NW * 64) {
+      const int row = e / (NCOL / Q), col = e % (NCOL / Q) * Q;
       const int n = bx * NCOL + col;
       if (n >= N) continue;
-      float s = 0.f;
+      float sum[Q];
+      wave_sums(row, col, sum);
+      if constexpr (Q == 4) {  // (N is a multiple of 8 and the host checks the buffer's alignment)
+        *reinterpret_cast<floatx4*>(mine + (size_t)row * N + n) = floatx4{sum[0], sum[1], sum[2], sum[3]};
+      } else {
+        mine[(size_t)row * N + n] = sum[0];
+      }
+    }
+    return;
+  }
+  if (Q == 4 && ep.rope_d <= 0) {
+    // plain epilogue, a quad per thread
+    const bool out8 = (reinterpret_cast<uintptr_t>(out) & 7) == 0;  // the quad can go out as 8 bytes
+    for (int e = threadIdx.x; e < rows * (NCOL / Q); e += NW * 64) {
+      const int row = e / (NCOL / Q), col = e % (NCOL / Q) * Q;
+      const int n = bx * NCOL + col;
+      if (n >= N) continue;  // (N is a multiple of 8: a quad is inside or outside as a whole)
+      float sum[Q];
+      wave_sums(row, col, sum);
+      const size_t o = (size_t)(m_base + row) * N + n;
+      _Float16 res[Q];
 #pragma unroll
-      for (int w = 0; w < NW; ++w) s += red[w][row][col];
-      mine[(size_t)row * N + n] = s;
+      for (int c = 0; c < Q; ++c) {
+        float v = sum[c];
+        if (bias) v += (float)bias[n + c];
+        if (ep.gelu) {  // gelu_new, see below
+          const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+          v = v / (1.0f + __expf(-2.0f * u));
+        }
+        if (ep.add0) v += (float)reinterpret_cast<const _Float16*>(ep.add0)[o + c];
+        if (ep.add1) v += (float)reinterpret_cast<const _Float16*>(ep.add1)[o + c];
+        res[c] = (_Float16)v;
+      }
+      if (out8) {
+        typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<half4*>(out + o) = half4{res[0], res[1], res[2], res[3]};
+      } else {
+#pragma unroll
+        for (int c = 0; c < Q; ++c) out[o + c] = res[c];
+      }
     }
     return;
   }
@@ -618,7 +690,7 @@ int prepare(const xmk::Int4Call& c, int64_t m, int64_t group, Config* cfg) {
   }
   cfg->ksplit = 1;
   if (c.split.ksplit > 1) {
-    if (m > 16 || !c.split.partial || c.split.ksplit > xmk::kInt4MaxSplit ||
+    if (m > 16 || !c.split.partial || !xmk::aligned(c.split.partial, 16) || c.split.ksplit > xmk::kInt4MaxSplit ||
         c.split.partial_bytes < (size_t)c.split.ksplit * 32 * n * sizeof(float))
       return xmk::fail(XMK_INTERNAL, "int4_gemm: bad K split request");
     cfg->w = 4;
