@@ -70,6 +70,9 @@ def test_int4_gemm_gptj_mlp_shape(xmk, oracle, m):
     (10, 9216, 264, 128, True), (5, 5632, 136, 64, False), (30, 9216, 72, 128, False),
     # more than 256 column blocks with 2 to 16 rows: four-wave work-groups (ragged last block; 9 groups over 4 waves)
     (4, 512, 16640, 128, True), (12, 256, 16448, 64, False), (6, 1152, 16400, 128, True), (3, 128, 16392, 32, False),
+    # 16 groups per wave with the activations staged through LDS (eight-wave and four-wave forms): the reads of
+    # both staging buffers inside the loop have to wait for their loads
+    (32, 16384, 1024, 128, False), (6, 8192, 16400, 128, True),
     # groups of 256 channels run as two batches of 128 with the same scale and zero point
     (1, 2048, 512, 256, True), (8, 1024, 264, 256, False), (32, 4096, 256, 256, True), (4, 4096, 4096, 256, False),
 ])
