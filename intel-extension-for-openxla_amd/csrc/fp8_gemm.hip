@@ -209,7 +209,10 @@ __global__ __launch_bounds__(WGM * WGN * 64) void fp8_gemm_kernel(Fp8Params p) {
       else fa[0] = fa_addr.read(nxt, 0);
       if constexpr (i < TN) fb[par ^ 1][i] = fb_addr.read(nxt + A_BYTES, i);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = mfma_fp8(fb[par][j], fa[i & 1], acc[i][j]);
+      for (int j = 0; j < TN; ++j) {
+        const int jj = (i & 1) ? TN - 1 - j : j;  // boustrophedon: consecutive MFMAs share one operand
+        acc[i][jj] = mfma_fp8(fb[par][jj], fa[i & 1], acc[i][jj]);
+      }
     });
     // Issue order: each row of MFMAs starts with its LDS reads (4 x 16 bytes), the global loads
     // are spread evenly.

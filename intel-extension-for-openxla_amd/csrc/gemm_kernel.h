@@ -515,7 +515,10 @@ __global__ __launch_bounds__(WGM * WGN * 64) void gemm_mfma_kernel(GemmParams p)
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = Elem<T>::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
+      for (int j = 0; j < TN; ++j) {
+        const int jj = (i & 1) ? TN - 1 - j : j;  // boustrophedon: consecutive MFMAs share one operand
+        acc[i][jj] = Elem<T>::mfma(fb[buf][jj], fa[buf][i], acc[i][jj]);
+      }
   };
   constexpr int READS = (A_MC ? 2 : 1) * TM + (B_MC ? 2 : 1) * TN;
   constexpr int NMFMA = TM * TN;
