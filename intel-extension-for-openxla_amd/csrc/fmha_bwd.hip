@@ -159,24 +159,22 @@ int run(const void* q, const void* k, const void* v, const void* bias, const voi
   const int64_t rows = units * F;
   const bool fused = fused_path((uint64_t)units, (uint32_t)H, (uint32_t)F, (uint32_t)Tk, bias != nullptr);
   float* lse2 = reinterpret_cast<float*>(ws + dsum_bytes((uint64_t)units, (uint64_t)F));  // fused path only
+  // The gradients come from the fused kernels, which keep the scores on chip and form the two per-row
+  // statistics (D, LSE log2(e)) themselves; XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
+  if (fused) {
+    const fmha_bwd_fused::Args a{q, k, v, d_o, o, bias, lse, lse2, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
+    fmha_bwd_fused::launch(a, (uint64_t)units, dtype == XMK_BF16, st);
+    return xmk::check_launch("fmha_bwd");
+  }
   if (H <= 64)
     hipLaunchKernelGGL((dp_sum_kernel<T, 8>), dim3((unsigned)xmk::ceil_div(rows, 32)), dim3(256), 0, st, (const T*)o, dO,
-                       dsum, rows, (int)H, fused ? lse : nullptr, fused ? lse2 : nullptr);
+                       dsum, rows, (int)H, (const float*)nullptr, (float*)nullptr);
   else if (H <= 128)
     hipLaunchKernelGGL((dp_sum_kernel<T, 16>), dim3((unsigned)xmk::ceil_div(rows, 16)), dim3(256), 0, st, (const T*)o, dO,
-                       dsum, rows, (int)H, fused ? lse : nullptr, fused ? lse2 : nullptr);
+                       dsum, rows, (int)H, (const float*)nullptr, (float*)nullptr);
   else
     hipLaunchKernelGGL((dp_sum_kernel<T, 32>), dim3((unsigned)xmk::ceil_div(rows, 8)), dim3(256), 0, st, (const T*)o, dO,
-                       dsum, rows, (int)H, fused ? lse : nullptr, fused ? lse2 : nullptr);
-  // The gradients come from the fused kernels, which keep the scores on chip;
-  // XMK_FMHA_BWD_COMPOSED=1 forces the GEMM composition below.
-  {
-    const fmha_bwd_fused::Args a{q, k, v, d_o, bias, lse2, dsum, dq, dk, dv, (int)H, (int)F, (int)Tk, scale, causal != 0};
-    if (fused) {
-      fmha_bwd_fused::launch(a, (uint64_t)units, dtype == XMK_BF16, st);
-      return xmk::check_launch("fmha_bwd");
-    }
-  }
+                       dsum, rows, (int)H, (const float*)nullptr, (float*)nullptr);
   const int64_t ldT = pl.ldT, sst = F * ldT;  // score buffers: row length, unit stride
   int rc;
   for (int64_t u0 = 0; u0 < units; u0 += pl.chunk) {

@@ -12,9 +12,11 @@ struct Args {
   const void* k;
   const void* v;
   const void* d_o;
-  const void* bias;   // [units, F, T] additive bias or null
-  const float* lse;   // [units, F] log-sum-exp of the forward pass times log2(e)
-  const float* dsum;  // [units, F] rowsum(dO o O)
+  const void* o;         // [units, F, H] output of the forward pass
+  const void* bias;      // [units, F, T] additive bias or null
+  const float* lse_fwd;  // [units, F] log-sum-exp of the forward pass
+  float* lse;            // scratch [units, F]: LSE times log2(e)       } written by the queries-own launch,
+  float* dsum;           // scratch [units, F]: D = rowsum(dO o O)       } read by the keys-own launches after it
   void* dq;
   void* dk;
   void* dv;
@@ -25,7 +27,7 @@ struct Args {
 
 // Head sizes up to 256 (multiples of 8); a bias of at most 2 GiB per unit.
 bool eligible(const Args& a, uint64_t units);
-// Two launches: keys own (dK, dV), then queries own (dQ).
+// Queries own (dQ; it also forms the two per-row statistics), then keys own (dK, dV).
 void launch(const Args& a, uint64_t units, bool bf16, hipStream_t stream);
 
 }  // namespace fmha_bwd_fused

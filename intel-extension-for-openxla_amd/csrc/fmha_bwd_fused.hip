@@ -81,8 +81,10 @@ struct KParams {
   const void* strm2;  // streamed operand of the dP product:    dO (owner = keys) or V
   const void* bias;   // [units, F, T] additive bias of the scores, or null
   int bias_vec;       // queries-own pass: the bias may be read 4 keys (8 bytes) at a time
-  const float* lse;   // [units, F] LSE of the forward pass times log2(e)
-  const float* dsum;  // [units, F] D = rowsum(dO o O)
+  float* lse;         // [units, F] LSE of the forward pass times log2(e)    } the queries-own launch writes them,
+  float* dsum;        // [units, F] D = rowsum(dO o O)                       } the keys-own launches read them
+  const void* o;      // [units, F, H] forward output and
+  const float* lse_fwd;  // [units, F] its LSE (queries-own launch)
   void* out1;         // scale * dS^T Q (dK)  or  scale * dS K (dQ)
   void* out2;         // P^T dO (dV), owner = keys only
   int H, F, T;
@@ -152,8 +154,8 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
   const T* Own2 = reinterpret_cast<const T*>(p.own2) + (int64_t)unit * n_own * H;
   const T* Str1 = reinterpret_cast<const T*>(p.strm1) + (int64_t)unit * n_str * H;
   const T* Str2 = reinterpret_cast<const T*>(p.strm2) + (int64_t)unit * n_str * H;
-  const float* lse = p.lse + (int64_t)unit * p.F;
-  const float* dsum = p.dsum + (int64_t)unit * p.F;
+  float* lse = p.lse + (int64_t)unit * p.F;
+  float* dsum = p.dsum + (int64_t)unit * p.F;
 
   // ---- owner fragments (B operands): this wave holds owner rows wo0 + l%32, fragment s covers
   // h = 16 s + 8 g .. +7.
@@ -172,12 +174,33 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
       if constexpr (DS) of2[s] = __builtin_bit_cast(V8, buf_load(r2, off));
     }
   }
-  // Softmax statistics of the lane's own query row (owner = queries).
+  // Softmax statistics of the lane's own query row (owner = queries): LSE log2(e) (one multiplication per row here
+  // instead of one per score) and D = sum_h O[row][h] dO[row][h] (fmha_backward.h:48), formed from the dO fragments
+  // the wave holds anyway and the same pieces of O, and written out for the keys-own launches that follow: a
+  // separate pass over O and dO for them was 45 us at [8,32,2048,128].
   float own_lse2 = 0.f, own_d = 0.f;
   if constexpr (!OWNER_K) {
+    static_assert(DS, "the queries-own launch holds dO");
+    const T* Oo = reinterpret_cast<const T*>(p.o) + (int64_t)unit * n_own * H;
+    const __amdgpu_buffer_rsrc_t ro = make_rsrc(Oo + (int64_t)o0 * H, (uint32_t)(n_own - o0) * H * 2);
+    float part = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int h = 16 * s + 8 * g;
+      const uint32_t off = h < H ? (uint32_t)(((wave * 32 + l32) * H + h) * 2) : kOob;
+      const u32x4 ow = buf_load(ro, off);
+      const T* oe = reinterpret_cast<const T*>(&ow);
+      const T* de = reinterpret_cast<const T*>(&of2[s]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part += (float)oe[e] * (float)de[e];
+    }
+    own_d = part + __shfl_xor(part, 32);  // the row's other eight-element pieces are in lane l ^ 32
     if (orow < p.F) {
-      own_lse2 = lse[orow];
-      own_d = dsum[orow];
+      own_lse2 = p.lse_fwd[(int64_t)unit * p.F + orow] * 1.4426950408889634f;
+      if (g == 0) {
+        lse[orow] = own_lse2;
+        dsum[orow] = own_d;
+      }
     }
   }
 
@@ -480,10 +503,13 @@ void launch_pass(KParams p, uint64_t units, bool causal, hipStream_t st) {
 template <typename T, int HP>
 void launch_both(const fmha_bwd_fused::Args& a, uint64_t units, hipStream_t st) {
   KParams p;
-  p.lse = a.lse; p.dsum = a.dsum; p.H = a.H; p.F = a.F; p.T = a.T; p.scale = a.scale;
+  p.lse = a.lse; p.dsum = a.dsum; p.o = a.o; p.lse_fwd = a.lse_fwd; p.H = a.H; p.F = a.F; p.T = a.T; p.scale = a.scale;
   p.bias = a.bias;
   p.bias_vec = a.bias && a.T % 4 == 0 && xmk::aligned(a.bias, 8);
   p.nob = p.total = p.per_xcd = 0;
+  // owner = queries first: dQ, and the per-row statistics the other launches read
+  p.own1 = a.q; p.own2 = a.d_o; p.strm1 = a.k; p.strm2 = a.v; p.out1 = a.dq; p.out2 = nullptr;
+  launch_pass<T, HP, false, true, false>(p, units, a.causal, st);
   // owner = keys: dK, then dV
   p.own1 = a.k; p.own2 = a.v; p.strm1 = a.q; p.strm2 = a.d_o; p.out1 = a.dk; p.out2 = a.dv;
   // One pass for both where the two accumulators fit beside everything else (S is then computed once for the
@@ -496,9 +522,6 @@ void launch_both(const fmha_bwd_fused::Args& a, uint64_t units, hipStream_t st) 
     launch_pass<T, HP, true, true, false>(p, units, a.causal, st);
     launch_pass<T, HP, true, false, true>(p, units, a.causal, st);
   }
-  // owner = queries: dQ
-  p.own1 = a.q; p.own2 = a.d_o; p.strm1 = a.k; p.strm2 = a.v; p.out1 = a.dq; p.out2 = nullptr;
-  launch_pass<T, HP, false, true, false>(p, units, a.causal, st);
 }
 
 }  // namespace
