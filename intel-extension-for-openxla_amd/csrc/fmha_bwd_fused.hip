@@ -161,49 +161,10 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
   // h = 16 s + 8 g .. +7.
   const int wo0 = o0 + wave * 32;
   const int orow = wo0 + l32;
+  // They come in through LDS like the streamed tiles (below, once the tile loader is set up): read from global
+  // memory in this layout, neighbouring lanes hold different rows, every lane is a cache access of its own, and
+  // eight such loads per wave and operand cost the launch 18 us of load-path time at [8,32,2048,128].
   V8 of1[KS], of2[KS];
-  {
-    const int rows_left = n_own - o0;  // > 0
-    const __amdgpu_buffer_rsrc_t r1 = make_rsrc(Own1 + (int64_t)o0 * H, (uint32_t)rows_left * H * 2);
-    const __amdgpu_buffer_rsrc_t r2 = make_rsrc(Own2 + (int64_t)o0 * H, (uint32_t)rows_left * H * 2);
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int h = 16 * s + 8 * g;
-      const uint32_t off = h < H ? (uint32_t)(((wave * 32 + l32) * H + h) * 2) : kOob;  // rows past the end are out of range
-      of1[s] = __builtin_bit_cast(V8, buf_load(r1, off));
-      if constexpr (DS) of2[s] = __builtin_bit_cast(V8, buf_load(r2, off));
-    }
-  }
-  // Softmax statistics of the lane's own query row (owner = queries): LSE log2(e) (one multiplication per row here
-  // instead of one per score) and D = sum_h O[row][h] dO[row][h] (fmha_backward.h:48), formed from the dO fragments
-  // the wave holds anyway and the same pieces of O, and written out for the keys-own launches that follow: a
-  // separate pass over O and dO for them was 45 us at [8,32,2048,128].
-  float own_lse2 = 0.f, own_d = 0.f;
-  if constexpr (!OWNER_K) {
-    static_assert(DS, "the queries-own launch holds dO");
-    const T* Oo = reinterpret_cast<const T*>(p.o) + (int64_t)unit * n_own * H;
-    const __amdgpu_buffer_rsrc_t ro = make_rsrc(Oo + (int64_t)o0 * H, (uint32_t)(n_own - o0) * H * 2);
-    float part = 0.f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int h = 16 * s + 8 * g;
-      const uint32_t off = h < H ? (uint32_t)(((wave * 32 + l32) * H + h) * 2) : kOob;
-      const u32x4 ow = buf_load(ro, off);
-      const T* oe = reinterpret_cast<const T*>(&ow);
-      const T* de = reinterpret_cast<const T*>(&of2[s]);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) part += (float)oe[e] * (float)de[e];
-    }
-    own_d = part + __shfl_xor(part, 32);  // the row's other eight-element pieces are in lane l ^ 32
-    if (orow < p.F) {
-      own_lse2 = p.lse_fwd[(int64_t)unit * p.F + orow] * 1.4426950408889634f;
-      if (g == 0) {
-        lse[orow] = own_lse2;
-        dsum[orow] = own_d;
-      }
-    }
-  }
-
   // ---- streamed tile loads, global -> LDS, as in the forward kernel: load j = i * NW + wave fills
   // LDS bytes [1024 j, +1024) of the tile; lane l lands at row j * RPL + l / CPR, chunk l % CPR, and
   // fetches the global chunk that belongs there under the swizzle (swz below).
@@ -216,8 +177,8 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
     koff[v] = chunk * 8 < H ? (uint32_t)((lrow * H + chunk * 8) * 2) : kOob;
   }
   const uint32_t lstride = (uint32_t)(LROWS * H * 2);
-  auto issue_tile = [&](const T* base, int t0, char* __restrict__ tile) {
-    const int rows_left = n_str - t0;  // > 0
+  auto issue_rows = [&](const T* base, int t0, char* __restrict__ tile, int n_rows) {
+    const int rows_left = n_rows - t0;  // (<= 0: the whole tile is zeros)
     const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)t0 * H, 0x7fffffffu);
     const bool full = rows_left >= BS;
 #pragma unroll
@@ -227,6 +188,7 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
                                                i * lstride, 0, 0);
     }
   };
+  auto issue_tile = [&](const T* base, int t0, char* __restrict__ tile) { issue_rows(base, t0, tile, n_str); };
   // LSE (waves 0, 2) and D (waves 1, 3) of the block's 64 query rows, one float per lane; rows past
   // F load zeros.  Every wave issues one load so that the load counts stay uniform.
   auto issue_stats = [&](int t0, char* __restrict__ st) {
@@ -350,6 +312,59 @@ __global__ __launch_bounds__(256, (HP <= 128 && !BIAS && !(DS && PV && HP > 64))
   char* const s1 = lds;              // streamed tiles of the score product, two stages
   char* const s2 = lds + 2 * TILE;   // streamed tiles of the dP product, two stages
   char* const sst = lds + 4 * TILE;  // statistics, two stages
+
+  // ---- owner fragments: the block's BO = 2 BS owner rows of each operand fill the two stages of s1 / s2; wave w
+  // picks its 32 rows' fragments up as row fragments of tile w / 2, half w % 2.
+  static_assert(BO == 2 * BS, "an owner block fills both stages");
+  const char* const own_at = lds + (wave >> 1) * TILE + (wave & 1) * 32 * ROWB;
+  issue_rows(Own1, o0, s1, n_own);
+  issue_rows(Own1, o0 + BS, s1 + TILE, n_own);
+  if constexpr (DS) {
+    issue_rows(Own2, o0, s2, n_own);
+    issue_rows(Own2, o0 + BS, s2 + TILE, n_own);
+  }
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    of1[s] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(own_at + kbase[s]));
+    if constexpr (DS) of2[s] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(own_at + 2 * TILE + kbase[s]));
+  }
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+  __builtin_amdgcn_s_barrier();  // every wave has its fragments: the stages may be overwritten
+  // Softmax statistics of the lane's own query row (owner = queries): LSE log2(e) (one multiplication per row here
+  // instead of one per score) and D = sum_h O[row][h] dO[row][h] (fmha_backward.h:48), formed from the dO fragments
+  // the wave holds anyway and the same pieces of O, and written out for the keys-own launches that follow: a
+  // separate pass over O and dO for them was 45 us at [8,32,2048,128].
+  float own_lse2 = 0.f, own_d = 0.f;
+  if constexpr (!OWNER_K) {
+    static_assert(DS, "the queries-own launch holds dO");
+    const T* Oo = reinterpret_cast<const T*>(p.o) + (int64_t)unit * n_own * H;
+    issue_rows(Oo, o0, s1, n_own);
+    issue_rows(Oo, o0 + BS, s1 + TILE, n_own);
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+    __builtin_amdgcn_s_barrier();
+    float part = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const u32x4 ow = *reinterpret_cast<const u32x4*>(own_at + kbase[s]);
+      const T* oe = reinterpret_cast<const T*>(&ow);
+      const T* de = reinterpret_cast<const T*>(&of2[s]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part += (float)oe[e] * (float)de[e];
+    }
+    own_d = part + __shfl_xor(part, 32);  // the row's other eight-element pieces are in lane l ^ 32
+    if (orow < p.F) {
+      own_lse2 = p.lse_fwd[(int64_t)unit * p.F + orow] * 1.4426950408889634f;
+      if (g == 0) {
+        lse[orow] = own_lse2;
+        dsum[orow] = own_d;
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(0));
+    __builtin_amdgcn_s_barrier();
+  }
+
 
   // One block: its tiles are in `c1`, `c2`, `cst`; the next block's go to `n1`, `n2`, `nst`.
   auto block = [&](int it, const char* __restrict__ c1, const char* __restrict__ c2, const char* __restrict__ cst,
