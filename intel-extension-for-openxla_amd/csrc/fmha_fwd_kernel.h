@@ -196,18 +196,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   // h = 16 s + 8 g .. +7.
   const int wq0 = q0 + wave * 32;
   const int qrow = wq0 + l32;
+  // They come in through LDS (prologue below): read from global memory in this layout, neighbouring lanes hold
+  // different rows and every lane is a cache access of its own, four times the load-path time of a tile load.
   V8 qf[KS];
-  {
-    const int rows_left = F - q0;  // > 0
-    const __amdgpu_buffer_rsrc_t rq = make_rsrc(Q + (int64_t)q0 * H, (uint32_t)rows_left * H * 2);
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int h = 16 * s + 8 * g;
-      const int r = wave * 32 + l32;
-      const uint32_t off = h < H ? (uint32_t)((r * H + h) * 2) : kOob;  // rows past F are out of range
-      qf[s] = __builtin_bit_cast(V8, buf_load(rq, off));
-    }
-  }
 
   // ---- K / V half-tile loads, global -> LDS.  Load j = i * NW + wave fills LDS bytes [1024 j, +1024)
   // of the stage, i.e. half-tile rows j * RPL ..; lane l lands at row j * RPL + l / CPR, chunk l % CPR,
@@ -254,6 +245,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(stage + (i * NW + wave) * 1024), 16, off,
                                                  i * lstride, 0, 0);
       }
+    }
+  };
+
+  // The 32 query rows of wave i as a half tile in K's layout (rows past F: zeros).
+  auto issue_q = [&](int i_half, char* __restrict__ stage) {
+    const int rows_left = F - q0 - 32 * i_half;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(Q + (int64_t)(q0 + 32 * i_half) * H, 0x7fffffffu);
+    const bool full = rows_left >= 32;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const uint32_t off = (full || lrow + i * LROWS < rows_left) ? koff[i % KV] : kOob;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_ptr)(stage + (i * NW + wave) * 1024), 16, off, i * lstride, 0, 0);
     }
   };
 
@@ -615,10 +618,21 @@ __global__ __launch_bounds__(NW * 64, WPS) void fmha_fwd_kernel(FmhaParams p) {
   typedef std::integral_constant<int, 2> hs2;
   typedef std::integral_constant<int, 3> hs3;
 
-  // Prologue: the first two K half tiles, then the four half tiles the pipeline keeps ahead.
+  // Prologue: the query rows, staged in the V ring (free until V half tile 0 is sent) and read back as row
+  // fragments, wave w those of stage w; beside them the first two K half tiles, then the four half tiles the
+  // pipeline keeps ahead.
+  static_assert(NW <= NST, "one V stage per wave for the query rows");
+#pragma unroll
+  for (int i = 0; i < NW; ++i) issue_q(i, vst0 + i * HALF);
   if constexpr (BIAS == 2) issue_bias(0, btile);
   issue_half(false_type{}, K, 0, kst0, koff, KV);
   issue_half(false_type{}, K, 1, kst0 + HALF, koff, KV);
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(2 * NL + (BIAS == 2 ? 4 : 0)));  // the query rows have landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int s = 0; s < KS; ++s) qf[s] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(vst0 + wave * HALF + kbase[s]));
+  __builtin_amdgcn_s_waitcnt(wait_vm_lgkm0(63));  // (lgkmcnt(0): the fragments are in registers)
+  __builtin_amdgcn_s_barrier();                   // every wave has its own: the V ring may be filled
   issue_half(false_type{}, V, 0, vst0, &voff, 1);
   issue_half(true_type{}, K, 2, kst0 + 2 * HALF, koff, KV);  // (ranged: past the keys they touch no memory, and
   issue_half(true_type{}, K, 3, kst0 + 3 * HALF, koff, KV);  //  the count of loads in flight is the same for every T)
